@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused attention-JVP forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch: the fused forward (O, TO, lse, mu) followed by
+the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
+B=64, H=12, L=128, D=64, bf16 inputs / fp32 accumulation, q,k,v ~ N(0,1)*0.5, tangents ~ N(0,1)*0.1,
+cotangents ~ N(0,1), seed 0, inputs resident in HBM.  Throughput uses the work model
+42*B*H*L^2*D flop per step (forward 6 + backward 15 tile contractions).  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "JVP-attn fwd+bwd TFLOP/s, % bf16 MFMA peak (B=64,H=12,L=128,D=64)"
+B, H, L, D = 64, 12, 128, 64
+PRIMAL_SCALE, TANGENT_SCALE, SEED = 0.5, 0.1, 0
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
+
+
+def step_flops(b=B, h=H, l=L, d=D) -> float:
+    return 42.0 * b * h * l * l * d
+
+
+def make_inputs(device, b=B):
+    """q,k,v,tq,tk,tv,dO,dTO from one CPU generator in this order (fp32 N(0,1), scaled, cast)."""
+    g = torch.Generator().manual_seed(SEED)
+    out = {}
+    for n in NAMES:
+        x = torch.randn(b, H, L, D, generator=g, dtype=torch.float32)
+        if n in ("q", "k", "v"):
+            x *= PRIMAL_SCALE
+        elif n in ("tq", "tk", "tv"):
+            x *= TANGENT_SCALE
+        out[n] = x.to(torch.bfloat16).to(device)
+    return out
+
+
+def cpu_baseline(seconds: float = 12.0):
+    """The reference's CPU math path (torch.func.jvp over eager softmax(QK^T s)V, then autograd for the
+    six gradients; oracle.attention_jvp_autograd in fp32) on a bounded sample of the same workload:
+    the first 8 of the 64 batches, bf16 inputs up-cast to fp32, all host threads torch uses."""
+    from oracle import attn_jvp_oracle as orc
+    sample_b = 8
+    x = make_inputs("cpu", b=sample_b)
+    args = [x[n] for n in NAMES]
+    run = lambda: orc.attention_jvp_autograd(*args, dtype=torch.float32)
+    run()
+    times = []
+    t_end = time.perf_counter() + seconds
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": step_flops(b=sample_b) / med / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"B={sample_b} of 64 (H=12,L=128,D=64), fp32 eager torch.func.jvp + autograd.grad, "
+                  f"median of {len(times)} runs, {med * 1e3:.1f} ms each",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build targets one GPU; run with --gpus 1 (no multi-GPU path exists: "
+              "every (batch, head) pair is an independent problem and shards without communication)",
+              file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (torch.cuda.is_available() is False)", file=sys.stderr)
+        return 2
+
+    from semicat_amd import _lib, kernels
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    x = make_inputs(dev)
+    q, k, v, tq, tk, tv, dO, dTO = (x[n] for n in NAMES)
+    Lr = kernels.stat_rows(L)
+    o, to = torch.empty_like(q), torch.empty_like(q)
+    lse = torch.empty((B, H, Lr), device=dev, dtype=torch.float32)
+    mu = torch.empty_like(lse)
+    grads = tuple(torch.empty_like(q) for _ in range(6))
+
+    def fwd():
+        kernels.attention_jvp_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False)
+
+    def bwd():
+        kernels.attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads)
+
+    def step():
+        fwd()
+        bwd()
+
+    stream = torch.cuda.Stream()  # default priority; graph capture needs a non-default stream
+    graph = None
+    with torch.cuda.stream(stream):
+        for _ in range(3):
+            step()
+        stream.synchronize()
+        if not a.no_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                step()
+        run = graph.replay if graph is not None else step
+
+        for _ in range(a.warmup):
+            run()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            run()
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+
+        # per-phase durations with events on the launch stream (separate region, eager launches)
+        def timed(fn, n=50):
+            for _ in range(5):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(n):
+                fn()
+            e1.record(stream)
+            e1.synchronize()
+            return e0.elapsed_time(e1) / n  # ms
+
+        fwd_ms = timed(fwd)
+        bwd_ms = timed(bwd)
+
+    ms_per_step = wall / a.steps * 1e3
+    tflops = step_flops() / (ms_per_step * 1e-3) / 1e12
+
+    # Roofline of the forward kernel (one launch = the whole fused forward): algorithmic flops
+    # 12*L^2*D and bytes 8*L*D*2 (+12*L of statistics) per (batch, head).
+    fwd_flops = 12.0 * B * H * L * L * D
+    fwd_bytes = B * H * (8.0 * L * D * 2 + 12.0 * L)
+    bwd_flops = 30.0 * B * H * L * L * D
+    bwd_bytes = B * H * (16.0 * L * D * 2 + 16.0 * L)
+    # the backward launches dominate the step; its algorithmic intensity (flop/B) decides the bound
+    ai = bwd_flops / bwd_bytes
+    ridge = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)
+    if ai < ridge:
+        achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": achieved / PEAK_HBM_GBPS, "traffic": None}
+    else:
+        achieved = bwd_flops / (bwd_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None}
+    roofline["kernel"] = "sjvp_bwd (rowstats + col + row launches)"
+    roofline["ms"] = bwd_ms
+    roofline["mfma_frac"] = bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+
+    out = {
+        "metric": METRIC,
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "config 2: LM1B-shaped DiT attention JVP fwd+bwd, B=64 H=12 L=128 D=64, "
+                               "bf16 in / fp32 acc, non-causal, both cotangents",
+                   "launch": "eager" if graph is None else "hip-graph replay of one fwd+bwd step",
+                   "flop_model": "42*B*H*L^2*D"},
+        "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
+        "fwd_ms": fwd_ms,
+        "bwd_ms": bwd_ms,
+        "fwd_tflops": fwd_flops / (fwd_ms * 1e-3) / 1e12,
+        "fwd_gbps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+        "roofline": roofline,
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,102 @@
+/*
+ * sjvp.h - C ABI of the MI355X (gfx950) fused attention-JVP kernels.
+ *
+ * The library is the drop-in for the three kernel-level entry points of olsdavis/semicat's
+ * semicat/jvp_utils (paths below are relative to that repository):
+ *
+ *   sjvp_fwd   replaces flash_attention_jvp_multihead_triton_kernel_wrapper
+ *              (semicat/jvp_utils/ryu_triton.py:295-422, kernel :73-291)
+ *   sjvp_bwd   replaces, in ONE call, both
+ *              flash_jvp_backward._flash_attn_backward   (cotangent on the tangent output,
+ *              semicat/jvp_utils/flash_jvp_backward.py:2293-2714) and
+ *              flash_attn_triton._flash_attn_backward    (cotangent on the primal output,
+ *              semicat/jvp_utils/flash_attn_triton.py:974-1093)
+ *
+ * Conventions
+ *   - Tensors are [B,H,L,D] views described by a base pointer and three element strides
+ *     (batch, head, sequence); the last dimension has unit stride (the reference asserts the same,
+ *     flash_jvp_backward.py:2321-2322).  q, tq, o, to, dO, dTO, dq, dtq have L = Lq; the k/v side has
+ *     L = Lk.  Any [B,S,H,D] caller layout is expressed through the strides.
+ *   - dtype: SJVP_BF16 or SJVP_FP16 for every tensor; accumulation and softmax are fp32.
+ *   - Row statistics lse / mu / li are fp32 [B,H,Lr] contiguous with Lr = ceil(Lq/128)*128
+ *     (ryu_triton.py:351-358); rows >= Lq receive log(Lk), 0, Lk.
+ *   - scale <= 0 selects the default 1/sqrt(D) (ryu_triton.py:324-325).
+ *   - The caller owns every buffer, including the workspace; the library allocates no device
+ *     memory, keeps no pointer after returning, has no mutable global state, enqueues on the given
+ *     hipStream_t (passed as void*) of the CURRENT device and returns without synchronising.
+ *   - Every function returns SJVP_OK (0) or a negative error code; nothing aborts or throws.
+ *     Argument errors are detected before anything is launched.
+ *   - Results are deterministic: no atomics are used.
+ */
+#ifndef SJVP_H
+#define SJVP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SJVP_VERSION 1
+
+enum sjvp_dtype { SJVP_BF16 = 0, SJVP_FP16 = 1 };
+
+enum sjvp_status {
+    SJVP_OK = 0,
+    SJVP_ERR_NULL = -1,      /* a required pointer is NULL                                   */
+    SJVP_ERR_SHAPE = -2,     /* B, H, Lq or Lk < 1, or sizes beyond the 32-bit index range   */
+    SJVP_ERR_HEAD_DIM = -3,  /* D < 16 (ryu_triton.py:319-322) or D > 128 (flash_jvp_backward.py:2318) */
+    SJVP_ERR_DTYPE = -4,     /* dtype is neither SJVP_BF16 nor SJVP_FP16                     */
+    SJVP_ERR_WORKSPACE = -5, /* workspace NULL or smaller than sjvp_bwd_workspace_bytes()    */
+    SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (hipGetLastError)           */
+    SJVP_ERR_COTANGENT = -7  /* sjvp_bwd called with both dO and dTO NULL                    */
+};
+
+/* Indices into the stride tables: strides[3*i + {0,1,2}] = (batch, head, sequence) strides in
+ * elements of tensor i. */
+enum sjvp_fwd_tensor { SJVP_F_Q = 0, SJVP_F_K, SJVP_F_V, SJVP_F_TQ, SJVP_F_TK, SJVP_F_TV, SJVP_F_O,
+                       SJVP_F_TO, SJVP_F_COUNT };
+enum sjvp_bwd_tensor { SJVP_B_Q = 0, SJVP_B_K, SJVP_B_V, SJVP_B_TQ, SJVP_B_TK, SJVP_B_TV, SJVP_B_O,
+                       SJVP_B_TO, SJVP_B_DO, SJVP_B_DTO, SJVP_B_DQ, SJVP_B_DK, SJVP_B_DV, SJVP_B_DTQ,
+                       SJVP_B_DTK, SJVP_B_DTV, SJVP_B_COUNT };
+
+/*
+ * Fused forward: O = softmax(Q K^T scale) V and its forward-mode tangent
+ *   TO = (P * (S_dot - mu)) V + P V_dot,   S_dot = scale (Q_dot K^T + Q K_dot^T),  mu = rowsum(P * S_dot)
+ * in one online-softmax pass, plus lse (the reference's M), mu (MU) and, if li != NULL, the
+ * exp-sum relative to the row maximum (LI).   Replaces ryu_triton.py:295-422.
+ * Primal-only mode: tq = tk = tv = to = mu = NULL computes O and lse only.
+ */
+int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+             const void* tv, void* o, void* to, float* lse, float* mu, float* li, int B, int H,
+             int Lq, int Lk, int D, const int64_t* strides /* [SJVP_F_COUNT*3] */, float scale,
+             int dtype, void* stream);
+
+/*
+ * Fused backward for cotangents dO (on O) and dTO (on TO); either may be NULL (treated as zero,
+ * its contractions are skipped), not both.  Fills dq, dk, dv and, when dTO != NULL, dtq, dtk, dtv.
+ * With dTO == NULL (the primal node of autograd, functional.py:261-268) tq, tk, tv, to, mu and the
+ * three tangent gradients may be NULL.  o, to, lse, mu are the forward's outputs.
+ * Replaces flash_jvp_backward.py:2293-2714 and flash_attn_triton.py:974-1093.
+ */
+int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+             const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+             const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq, void* dtk,
+             void* dtv, void* workspace, size_t workspace_bytes, int B, int H, int Lq, int Lk, int D,
+             const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
+
+/* Bytes of caller-provided device scratch sjvp_bwd needs (row sums sum_4 and sum_7 + delta, which
+ * the reference allocates itself at flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
+size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
+
+/* Static, NUL-terminated description of a status code. */
+const char* sjvp_strerror(int status);
+
+/* SJVP_VERSION the library was built with. */
+int sjvp_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SJVP_H */

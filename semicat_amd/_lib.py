@@ -1,0 +1,73 @@
+"""ctypes binding of libsjvp.so (C ABI in include/sjvp.h).  There is no fallback: if the library is
+missing or a call fails, an exception is raised."""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+from . import build as _build
+
+SJVP_BF16 = 0
+SJVP_FP16 = 1
+
+SJVP_OK = 0
+SJVP_ERR_NULL = -1
+SJVP_ERR_SHAPE = -2
+SJVP_ERR_HEAD_DIM = -3
+SJVP_ERR_DTYPE = -4
+SJVP_ERR_WORKSPACE = -5
+SJVP_ERR_LAUNCH = -6
+SJVP_ERR_COTANGENT = -7
+
+F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
+B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
+             "dq", "dk", "dv", "dtq", "dtk", "dtv")
+
+EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_workspace_bytes", "sjvp_strerror", "sjvp_version")
+
+_lock = threading.Lock()
+_lib = None
+
+
+class SjvpError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"sjvp status {status}: {message}")
+        self.status = status
+
+
+def load() -> ctypes.CDLL:
+    """Load the in-tree shared library (building it first only if it does not exist)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            path = _build.LIB_PATH
+            if not os.path.exists(path):
+                _build.build()
+            lib = ctypes.CDLL(path)
+            vp, fp, i, i64p = ctypes.c_void_p, ctypes.POINTER(ctypes.c_float), ctypes.c_int, \
+                ctypes.POINTER(ctypes.c_int64)
+            lib.sjvp_fwd.argtypes = [vp] * 8 + [vp] * 3 + [i] * 5 + [i64p, ctypes.c_float, i, vp]
+            lib.sjvp_fwd.restype = i
+            lib.sjvp_bwd.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [vp, ctypes.c_size_t] + [i] * 5 +
+                                     [i64p, ctypes.c_float, i, vp])
+            lib.sjvp_bwd.restype = i
+            lib.sjvp_bwd_workspace_bytes.argtypes = [i] * 6
+            lib.sjvp_bwd_workspace_bytes.restype = ctypes.c_size_t
+            lib.sjvp_strerror.argtypes = [i]
+            lib.sjvp_strerror.restype = ctypes.c_char_p
+            lib.sjvp_version.argtypes = []
+            lib.sjvp_version.restype = i
+            _lib = lib
+    return _lib
+
+
+def strerror(status: int) -> str:
+    return load().sjvp_strerror(status).decode()
+
+
+def check(status: int) -> None:
+    if status != SJVP_OK:
+        raise SjvpError(status, strerror(status))

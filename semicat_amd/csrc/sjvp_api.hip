@@ -1,0 +1,244 @@
+// C ABI of the attention-JVP library (declared in include/sjvp.h): argument validation, kernel
+// selection and launches.  No device memory is allocated or freed here and no state is kept.
+#include "../../include/sjvp.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+
+#include "sjvp_bwd.hpp"
+#include "sjvp_fwd.hpp"
+
+using namespace sjvp;
+
+namespace {
+
+inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+struct VecCheck {
+    bool ok = true;
+    void add(const void* p, const int64_t* s) {
+        if (!p) return;
+        ok = ok && aligned16(p) && (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0);
+    }
+};
+
+inline TensorView view(const void* p, const int64_t* s) {
+    return TensorView{static_cast<const elem_t*>(p), s[0], s[1], s[2]};
+}
+inline OutView out_view(void* p, const int64_t* s) {
+    return OutView{static_cast<elem_t*>(p), s[0], s[1], s[2]};
+}
+
+int check_common(int B, int H, int Lq, int Lk, int D, int dtype) {
+    if (dtype != SJVP_BF16 && dtype != SJVP_FP16) return SJVP_ERR_DTYPE;
+    if (B < 1 || H < 1 || Lq < 1 || Lk < 1) return SJVP_ERR_SHAPE;
+    if (D < 16 || D > 128) return SJVP_ERR_HEAD_DIM;
+    const int64_t blocks = (int64_t)B * H * ((int64_t)round_up(Lq > Lk ? Lq : Lk, 32) / 32);
+    if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
+    return SJVP_OK;
+}
+
+template <typename K>
+int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params) {
+    if (smem_bytes > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                smem_bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return SJVP_ERR_LAUNCH;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem_bytes, stream, params);
+    return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
+}
+
+template <typename T, int HD>
+int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
+    constexpr int BN = 64;
+    if (jvp) return launch(fwd_kernel<T, HD, BN, true>, grid, FwdSmem<HD, BN, true>::bytes, stream, p);
+    return launch(fwd_kernel<T, HD, BN, false>, grid, FwdSmem<HD, BN, false>::bytes, stream, p);
+}
+
+template <typename T>
+int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
+    if (p.D <= 32) return fwd_hd<T, 32>(p, grid, jvp, stream);
+    if (p.D <= 64) return fwd_hd<T, 64>(p, grid, jvp, stream);
+    return fwd_hd<T, 128>(p, grid, jvp, stream);
+}
+
+template <typename T, int HD, bool HAS_DO, bool HAS_G>
+int bwd_mode(const BwdParams& p, int BH, hipStream_t stream) {
+    int rc = launch(bwd_rowstats_kernel<T, HAS_DO, HAS_G>, BH * (p.Lr / 32), 0, stream, p);
+    if (rc != SJVP_OK) return rc;
+    const int col_grid = BH * p.k_blocks;
+    if constexpr (HD == 128) {
+        // two launches, each accumulating half of the head dimension (register budget)
+        constexpr int BM = 32;
+        using SM = ColSmem<HD, BM, HAS_DO, HAS_G>;
+        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 0, 2>, col_grid, SM::bytes, stream, p);
+        if (rc != SJVP_OK) return rc;
+        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 2, 2>, col_grid, SM::bytes, stream, p);
+    } else {
+        constexpr int BM = 64;
+        using SM = ColSmem<HD, BM, HAS_DO, HAS_G>;
+        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 0, HD / 32>, col_grid, SM::bytes, stream,
+                    p);
+    }
+    if (rc != SJVP_OK) return rc;
+    constexpr int BN = 64;
+    return launch(bwd_row_kernel<T, HD, BN, HAS_DO, HAS_G>, BH * p.q_blocks,
+                  RowSmem<HD, BN, HAS_G>::bytes, stream, p);
+}
+
+template <typename T, int HD>
+int bwd_hd(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
+    if (has_do && has_g) return bwd_mode<T, HD, true, true>(p, BH, stream);
+    if (has_g) return bwd_mode<T, HD, false, true>(p, BH, stream);
+    return bwd_mode<T, HD, true, false>(p, BH, stream);
+}
+
+template <typename T>
+int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
+    if (p.D <= 32) return bwd_hd<T, 32>(p, BH, has_do, has_g, stream);
+    if (p.D <= 64) return bwd_hd<T, 64>(p, BH, has_do, has_g, stream);
+    return bwd_hd<T, 128>(p, BH, has_do, has_g, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+             const void* tv, void* o, void* to, float* lse, float* mu, float* li, int B, int H,
+             int Lq, int Lk, int D, const int64_t* strides, float scale, int dtype, void* stream) {
+    if (!q || !k || !v || !o || !lse || !strides) return SJVP_ERR_NULL;
+    const bool jvp = tq || tk || tv || to || mu;
+    if (jvp && (!tq || !tk || !tv || !to || !mu)) return SJVP_ERR_NULL;
+    int rc = check_common(B, H, Lq, Lk, D, dtype);
+    if (rc != SJVP_OK) return rc;
+
+    const void* ptrs[SJVP_F_COUNT] = {q, k, v, tq, tk, tv, o, to};
+    VecCheck vc;
+    for (int i = 0; i < SJVP_F_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
+
+    FwdParams p{};
+    p.q = view(q, strides + 3 * SJVP_F_Q);
+    p.k = view(k, strides + 3 * SJVP_F_K);
+    p.v = view(v, strides + 3 * SJVP_F_V);
+    if (jvp) {
+        p.tq = view(tq, strides + 3 * SJVP_F_TQ);
+        p.tk = view(tk, strides + 3 * SJVP_F_TK);
+        p.tv = view(tv, strides + 3 * SJVP_F_TV);
+        p.to = static_cast<elem_t*>(to);
+        p.to_sb = strides[3 * SJVP_F_TO];
+        p.to_sh = strides[3 * SJVP_F_TO + 1];
+        p.to_sl = strides[3 * SJVP_F_TO + 2];
+    }
+    p.o = static_cast<elem_t*>(o);
+    p.o_sb = strides[3 * SJVP_F_O];
+    p.o_sh = strides[3 * SJVP_F_O + 1];
+    p.o_sl = strides[3 * SJVP_F_O + 2];
+    p.lse = lse;
+    p.mu = mu;
+    p.li = li;
+    p.H = H;
+    p.Lq = Lq;
+    p.Lk = Lk;
+    p.D = D;
+    p.Lr = round_up(Lq, 128);
+    p.q_blocks = p.Lr / 128;
+    p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+    p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
+
+    const int grid = B * H * p.q_blocks;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == SJVP_BF16 ? fwd_dtype<Bf16>(p, grid, jvp, s) : fwd_dtype<Fp16>(p, grid, jvp, s);
+}
+
+size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype) {
+    (void)Lk;
+    (void)D;
+    (void)dtype;
+    if (B < 1 || H < 1 || Lq < 1) return 0;
+    return (size_t)2 * (size_t)B * (size_t)H * (size_t)round_up(Lq, 128) * sizeof(float);
+}
+
+int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+             const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+             const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq, void* dtk,
+             void* dtv, void* workspace, size_t workspace_bytes, int B, int H, int Lq, int Lk, int D,
+             const int64_t* strides, float scale, int dtype, void* stream) {
+    if (!dO && !dTO) return SJVP_ERR_COTANGENT;
+    const bool has_do = dO != nullptr, has_g = dTO != nullptr;
+    if (!q || !k || !v || !o || !lse || !dq || !dk || !dv || !strides) return SJVP_ERR_NULL;
+    if (has_g && (!tq || !tk || !tv || !to || !mu || !dtq || !dtk || !dtv)) return SJVP_ERR_NULL;
+    int rc = check_common(B, H, Lq, Lk, D, dtype);
+    if (rc != SJVP_OK) return rc;
+    if (!workspace || workspace_bytes < sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype) ||
+        (reinterpret_cast<uintptr_t>(workspace) & 3u))
+        return SJVP_ERR_WORKSPACE;
+
+    const void* ptrs[SJVP_B_COUNT] = {q, k, v, has_g ? tq : nullptr, has_g ? tk : nullptr,
+                                      has_g ? tv : nullptr, o, has_g ? to : nullptr, dO, dTO, dq, dk,
+                                      dv, has_g ? dtq : nullptr, has_g ? dtk : nullptr,
+                                      has_g ? dtv : nullptr};
+    VecCheck vc;
+    for (int i = 0; i < SJVP_B_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
+
+    BwdParams p{};
+    p.q = view(q, strides + 3 * SJVP_B_Q);
+    p.k = view(k, strides + 3 * SJVP_B_K);
+    p.v = view(v, strides + 3 * SJVP_B_V);
+    p.o = view(o, strides + 3 * SJVP_B_O);
+    if (has_do) p.dO = view(dO, strides + 3 * SJVP_B_DO);
+    p.dq = out_view(dq, strides + 3 * SJVP_B_DQ);
+    p.dk = out_view(dk, strides + 3 * SJVP_B_DK);
+    p.dv = out_view(dv, strides + 3 * SJVP_B_DV);
+    if (has_g) {
+        p.tq = view(tq, strides + 3 * SJVP_B_TQ);
+        p.tk = view(tk, strides + 3 * SJVP_B_TK);
+        p.tv = view(tv, strides + 3 * SJVP_B_TV);
+        p.to = view(to, strides + 3 * SJVP_B_TO);
+        p.dTO = view(dTO, strides + 3 * SJVP_B_DTO);
+        p.dtq = out_view(dtq, strides + 3 * SJVP_B_DTQ);
+        p.dtk = out_view(dtk, strides + 3 * SJVP_B_DTK);
+        p.dtv = out_view(dtv, strides + 3 * SJVP_B_DTV);
+    }
+    p.lse = lse;
+    p.mu = mu;
+    p.H = H;
+    p.Lq = Lq;
+    p.Lk = Lk;
+    p.D = D;
+    p.Lr = round_up(Lq, 128);
+    p.q_blocks = p.Lr / 128;
+    p.k_blocks = round_up(Lk, 128) / 128;
+    p.s4 = static_cast<float*>(workspace);
+    p.s7d = p.s4 + (size_t)B * H * p.Lr;
+    p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+    p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, s)
+                              : bwd_dtype<Fp16>(p, B * H, has_do, has_g, s);
+}
+
+const char* sjvp_strerror(int status) {
+    switch (status) {
+        case SJVP_OK: return "ok";
+        case SJVP_ERR_NULL: return "a required pointer is NULL";
+        case SJVP_ERR_SHAPE: return "B, H, Lq and Lk must be >= 1 and within the index range";
+        case SJVP_ERR_HEAD_DIM: return "head dimension must satisfy 16 <= D <= 128";
+        case SJVP_ERR_DTYPE: return "dtype must be SJVP_BF16 or SJVP_FP16";
+        case SJVP_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than sjvp_bwd_workspace_bytes()";
+        case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
+        case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
+        default: return "unknown sjvp status";
+    }
+}
+
+int sjvp_version(void) { return SJVP_VERSION; }
+
+}  // extern "C"

@@ -1,0 +1,162 @@
+"""Autograd surface of the attention-JVP op: ``sdpa_jvp`` / ``safe_sdpa_jvp`` with the semantics of
+olsdavis/semicat's ``semicat/jvp_utils/functional.py`` (cited by line below), backed by the HIP
+kernels in :mod:`semicat_amd.kernels`.
+
+How the op is wired (same shape as the reference, functional.py:216-307):
+
+* ``SDPAFunction.forward`` only allocates the primal output ``y`` and the statistic ``M``
+  (functional.py:218-231); under forward-mode AD its ``jvp`` runs the fused kernel once, which
+  fills ``y`` and ``M`` in place and returns the tangent ``t_y`` (functional.py:240-258).
+* ``SDPAJVPForwardFunction`` is the reverse-mode node of the tangent output: its backward receives
+  the cotangent on ``t_y`` and returns gradients for q, k, v and the three tangents
+  (functional.py:52-87).
+* ``SDPAFunction.backward`` is the reverse-mode node of the primal output (functional.py:261-268).
+
+Beyond the reference: called without forward-mode tangents the reference returns an uninitialised
+``y`` (functional.py:286-287); here that case is detected and a primal-only kernel computes ``y``
+(and supports reverse mode), so the op is a strict superset.  A missing tangent is treated as zero.
+"""
+from __future__ import annotations
+
+from typing import Any, Optional
+
+import torch
+import torch.autograd.forward_ad as fwAD
+from torch import Tensor
+
+from . import kernels
+
+
+def _has_tangent(t: Tensor) -> bool:
+    return fwAD.unpack_dual(t).tangent is not None
+
+
+class SDPAJVPFlashBackwardFunction(torch.autograd.Function):
+    """Gradients for the cotangent on the tangent output (functional.py:90-168)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, t_q, t_k, t_v, tangents_t_o, lse, mu, o, t_o):
+        dq, dk, dv, dtq, dtk, dtv = kernels.attention_jvp_backward(
+            q, k, v, t_q, t_k, t_v, o, t_o, lse, mu, dO=None, dTO=tangents_t_o)
+        return dq, dk, dv, dtq, dtk, dtv
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("double backward of the attention-JVP op is not implemented")
+
+
+class SDPABackwardFunction(torch.autograd.Function):
+    """Gradients for the cotangent on the primal output (functional.py:171-213)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, o, do, M):
+        dq, dk, dv, _, _, _ = kernels.attention_jvp_backward(
+            q, k, v, None, None, None, o, None, M, None, dO=do, dTO=None)
+        return dq, dk, dv
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("double backward of the attention-JVP op is not implemented")
+
+
+class SDPAJVPForwardFunction(torch.autograd.Function):
+    """Runs the fused forward; node of the tangent output (functional.py:52-87)."""
+
+    @staticmethod
+    def forward(q, k, v, t_q, t_k, t_v, y, M):
+        # y and M (allocated by SDPAFunction.forward) are filled in place by the fused kernel.
+        # LI, which the reference also keeps (functional.py:57-59), is not needed by the backward.
+        with torch.no_grad():
+            _, t_y, _, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y, lse=M,
+                                                             with_li=False)
+        return t_y, MU
+
+    @staticmethod
+    def setup_context(ctx, inputs: tuple[Any, ...], output: Any) -> Any:
+        t_y, MU = output
+        ctx.save_for_backward(*inputs, t_y, MU)
+        ctx.mark_non_differentiable(MU)
+
+    @staticmethod
+    def backward(ctx, d_t_y, *args):
+        q, k, v, t_q, t_k, t_v, y, M, t_y, MU = ctx.saved_tensors
+        if d_t_y is None:
+            return (None,) * 8
+        grads = SDPAJVPFlashBackwardFunction.apply(q, k, v, t_q, t_k, t_v, d_t_y, M, MU, y, t_y)
+        return *grads, None, None
+
+
+class SDPAFunction(torch.autograd.Function):
+    """The op under forward-mode AD (functional.py:216-268)."""
+
+    @staticmethod
+    def forward(q, k, v):
+        B, H, S, D = q.shape
+        y = torch.empty((B, H, S, v.shape[-1]), device=q.device, dtype=q.dtype)
+        M = torch.empty((B, H, kernels.stat_rows(S)), device=q.device, dtype=torch.float32)
+        return y, M
+
+    @staticmethod
+    def setup_context(ctx: Any, inputs: tuple[Any, ...], output: Any) -> Any:
+        ctx.save_for_forward(*inputs, *output)
+        ctx.save_for_backward(*inputs, *output)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def jvp(ctx, t_q, t_k, t_v):
+        q, k, v, y, M = ctx.saved_for_forward
+        t_q = torch.zeros_like(q) if t_q is None else t_q
+        t_k = torch.zeros_like(k) if t_k is None else t_k
+        t_v = torch.zeros_like(v) if t_v is None else t_v
+        t_y, _ = SDPAJVPForwardFunction.apply(q, k, v, t_q, t_k, t_v, y, M)
+        return t_y, torch.zeros_like(M)
+
+    @staticmethod
+    def backward(ctx, d_y, d_M):
+        if d_y is None:
+            return None, None, None
+        q, k, v, y, M = ctx.saved_tensors
+        with torch.no_grad():
+            dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
+        return dq, dk, dv
+
+
+class SDPAPrimalFunction(torch.autograd.Function):
+    """The op without forward-mode tangents: plain attention with the primal-only kernels."""
+
+    @staticmethod
+    def forward(ctx, q, k, v):
+        y, M = kernels.attention_forward(q, k, v)
+        ctx.save_for_backward(q, k, v, y, M)
+        return y
+
+    @staticmethod
+    def backward(ctx, d_y):
+        q, k, v, y, M = ctx.saved_tensors
+        dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
+        return dq, dk, dv
+
+
+@torch._dynamo.disable
+def sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
+    """Fused scaled-dot-product attention with forward-mode (jvp) support; ``[B,H,S,D]`` bf16/fp16
+    (functional.py:272-307).  Usage: ``y, t_y = torch.func.jvp(sdpa_jvp, (q, k, v), (t_q, t_k, t_v))``
+    or wrap a whole model that calls it in ``torch.func.jvp``; both outputs support ``backward``."""
+    if _has_tangent(q) or _has_tangent(k) or _has_tangent(v):
+        y, _ = SDPAFunction.apply(q, k, v)
+        return y
+    return SDPAPrimalFunction.apply(q, k, v)
+
+
+def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
+    """``[B,S,H,D]`` wrapper that casts to bfloat16 when the inputs are neither bf16 nor fp16 and
+    casts the result back (functional.py:310-332)."""
+    orig_dtype = q.dtype
+    if orig_dtype != torch.bfloat16 and orig_dtype != torch.float16:
+        q = q.to(torch.bfloat16)
+        k = k.to(torch.bfloat16)
+        v = v.to(torch.bfloat16)
+    y = sdpa_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
+    if y.dtype != orig_dtype:
+        y = y.to(orig_dtype)
+    return y.transpose(1, 2)

@@ -1,0 +1,255 @@
+"""Kernel-level entry points: torch tensors in, HIP kernels (libsjvp.so, C ABI) launched on the
+current stream, nothing synchronised.  These replace the three launch wrappers of
+olsdavis/semicat's ``semicat/jvp_utils``:
+
+* :func:`flash_attention_jvp_multihead_kernel_wrapper`  <- ``ryu_triton.py:295-422``
+* :func:`flash_jvp_backward`                             <- ``flash_jvp_backward.py:2293-2714``
+* :func:`flash_attn_backward`                            <- ``flash_attn_triton.py:974-1093``
+
+plus the fused forms the autograd layer and the benchmark use (:func:`attention_jvp_forward`,
+:func:`attention_forward`, :func:`attention_jvp_backward`).  There is no CPU or eager fallback:
+tensors that are not on a GPU, or a missing shared library, raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16}
+
+
+def stat_rows(L: int) -> int:
+    """Length of the row-statistic buffers: L rounded up to 128 (ryu_triton.py:351)."""
+    return ((L + 127) // 128) * 128
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _strides(tensors: Sequence[Optional[torch.Tensor]]):
+    flat = []
+    for t in tensors:
+        flat.extend((0, 0, 0) if t is None else (t.stride(0), t.stride(1), t.stride(2)))
+    return (ctypes.c_int64 * len(flat))(*flat)
+
+
+def _check_bhld(name: str, t: torch.Tensor, shape, dtype, device) -> None:
+    if tuple(t.shape) != tuple(shape):
+        raise AssertionError(f"{name} shape mismatch: {tuple(t.shape)} != {tuple(shape)}")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} dtype {t.dtype} != {dtype}")
+    if t.device != device:
+        raise ValueError(f"{name} is on {t.device}, expected {device}")
+    if t.stride(-1) != 1:
+        raise AssertionError(f"{name}: the last dimension must have unit stride")
+
+
+def _require_gpu(q: torch.Tensor) -> int:
+    if not q.is_cuda:
+        raise RuntimeError("semicat_amd kernels run on an AMD GPU only; got a tensor on "
+                           f"{q.device} (there is no CPU fallback)")
+    if q.dtype not in _DTYPES:
+        raise TypeError(f"attention-JVP kernels support bfloat16 and float16, got {q.dtype}")
+    return _DTYPES[q.dtype]
+
+
+def _stat(buf: Optional[torch.Tensor], name: str, B: int, H: int, Lr: int, device) -> torch.Tensor:
+    if buf is None:
+        return torch.empty((B, H, Lr), device=device, dtype=torch.float32)
+    if tuple(buf.shape) != (B, H, Lr) or buf.dtype != torch.float32 or not buf.is_contiguous():
+        raise AssertionError(f"{name} must be a contiguous float32 tensor of shape {(B, H, Lr)}, "
+                             f"got {tuple(buf.shape)} {buf.dtype}")
+    return buf
+
+
+def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=None, to=None,
+                          lse=None, mu=None, li=None, with_li: bool = True
+                          ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                                     Optional[torch.Tensor]]:
+    """Fused forward on [B,H,L,D] views: returns (o, to, lse, mu, li); any of them may be passed in
+    to be filled in place.  ``with_li=False`` skips the LI statistic (returned as None)."""
+    dtype_tag = _require_gpu(q)
+    B, H, Lq, D = q.shape
+    Lk = k.shape[-2]
+    if D < 16:
+        raise ValueError(f"D_head must be >= 16, got {D}")
+    dev, dt = q.device, q.dtype
+    _check_bhld("Q", q, (B, H, Lq, D), dt, dev)
+    for name, t in (("K", k), ("V", v), ("t_K", tk), ("t_V", tv)):
+        _check_bhld(name, t, (B, H, Lk, D), dt, dev)
+    _check_bhld("t_Q", tq, (B, H, Lq, D), dt, dev)
+    if o is None:
+        o = torch.empty((B, H, Lq, D), device=dev, dtype=dt)
+    if to is None:
+        to = torch.empty((B, H, Lq, D), device=dev, dtype=dt)
+    _check_bhld("y", o, (B, H, Lq, D), dt, dev)
+    _check_bhld("t_y", to, (B, H, Lq, D), dt, dev)
+    Lr = stat_rows(Lq)
+    lse = _stat(lse, "M", B, H, Lr, dev)
+    mu = _stat(mu, "MU", B, H, Lr, dev)
+    li = _stat(li, "LI", B, H, Lr, dev) if (with_li or li is not None) else None
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.sjvp_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(tq), _ptr(tk), _ptr(tv), _ptr(o), _ptr(to),
+                          _ptr(lse), _ptr(mu), _ptr(li), B, H, Lq, Lk, D,
+                          _strides((q, k, v, tq, tk, tv, o, to)),
+                          float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+    _lib.check(rc)
+    return o, to, lse, mu, li
+
+
+def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
+                      ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Primal-only forward (tangent contractions compiled out): returns (o, lse)."""
+    dtype_tag = _require_gpu(q)
+    B, H, Lq, D = q.shape
+    Lk = k.shape[-2]
+    if D < 16:
+        raise ValueError(f"D_head must be >= 16, got {D}")
+    dev, dt = q.device, q.dtype
+    _check_bhld("Q", q, (B, H, Lq, D), dt, dev)
+    _check_bhld("K", k, (B, H, Lk, D), dt, dev)
+    _check_bhld("V", v, (B, H, Lk, D), dt, dev)
+    if o is None:
+        o = torch.empty((B, H, Lq, D), device=dev, dtype=dt)
+    _check_bhld("y", o, (B, H, Lq, D), dt, dev)
+    lse = _stat(lse, "M", B, H, stat_rows(Lq), dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.sjvp_fwd(_ptr(q), _ptr(k), _ptr(v), None, None, None, _ptr(o), None, _ptr(lse), None,
+                          None, B, H, Lq, Lk, D, _strides((q, k, v, None, None, None, o, None)),
+                          float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+    _lib.check(rc)
+    return o, lse
+
+
+def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
+                           scale: Optional[float] = None, grads=None):
+    """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
+    Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
+    tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
+    (the tangent three may be None without dTO)."""
+    dtype_tag = _require_gpu(q)
+    if dO is None and dTO is None:
+        raise ValueError("attention_jvp_backward needs a cotangent on o, on to, or on both")
+    B, H, Lq, D = q.shape
+    Lk = k.shape[-2]
+    if D > 128:
+        raise AssertionError(f"head dimension must be <= 128, got {D}")
+    dev, dt = q.device, q.dtype
+    has_g = dTO is not None
+    _check_bhld("q", q, (B, H, Lq, D), dt, dev)
+    _check_bhld("k", k, (B, H, Lk, D), dt, dev)
+    _check_bhld("v", v, (B, H, Lk, D), dt, dev)
+    _check_bhld("o", o, (B, H, Lq, D), dt, dev)
+    if dO is not None:
+        if dO.stride(-1) != 1:
+            dO = dO.contiguous()
+        _check_bhld("do", dO, (B, H, Lq, D), dt, dev)
+    if has_g:
+        if dTO.stride(-1) != 1:
+            dTO = dTO.contiguous()  # flash_jvp_backward.py:2314-2315
+        _check_bhld("dto", dTO, (B, H, Lq, D), dt, dev)
+        _check_bhld("tq", tq, (B, H, Lq, D), dt, dev)
+        _check_bhld("tk", tk, (B, H, Lk, D), dt, dev)
+        _check_bhld("tv", tv, (B, H, Lk, D), dt, dev)
+        _check_bhld("to", to, (B, H, Lq, D), dt, dev)
+    else:
+        tq = tk = tv = to = mu = None
+    Lr = stat_rows(Lq)
+    if tuple(lse.shape) != (B, H, Lr):
+        raise AssertionError(f"lse shape {tuple(lse.shape)} != {(B, H, Lr)}")
+    lse = _stat(lse, "lse", B, H, Lr, dev)
+    if has_g:
+        if mu.shape[-1] != Lr:  # flash_jvp_backward.py:2325-2339
+            mu = torch.cat([mu, mu.new_zeros((B, H, Lr - mu.shape[-1]))], dim=-1)
+        mu = _stat(mu.contiguous(), "mu", B, H, Lr, dev)
+    if grads is None:
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dtq, dtk, dtv = ((torch.empty_like(tq), torch.empty_like(tk), torch.empty_like(tv))
+                         if has_g else (None, None, None))
+    else:
+        dq, dk, dv, dtq, dtk, dtv = grads
+    _check_bhld("dq", dq, (B, H, Lq, D), dt, dev)
+    _check_bhld("dk", dk, (B, H, Lk, D), dt, dev)
+    _check_bhld("dv", dv, (B, H, Lk, D), dt, dev)
+    if has_g:
+        _check_bhld("dtq", dtq, (B, H, Lq, D), dt, dev)
+        _check_bhld("dtk", dtk, (B, H, Lk, D), dt, dev)
+        _check_bhld("dtv", dtv, (B, H, Lk, D), dt, dev)
+    else:
+        dtq = dtk = dtv = None
+    lib = _lib.load()
+    nbytes = lib.sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype_tag)
+    workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
+    tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.sjvp_bwd(*(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
+                          *(_ptr(t) for t in tensors[10:]), _ptr(workspace), nbytes, B, H, Lq, Lk, D,
+                          _strides(tensors), float(scale) if scale else 0.0, dtype_tag,
+                          ctypes.c_void_p(stream))
+    _lib.check(rc)
+    return dq, dk, dv, dtq, dtk, dtv
+
+
+# ------------------------------------------------------------------------------------------------
+# Drop-in replacements with the reference wrappers' own signatures.
+
+def flash_attention_jvp_multihead_kernel_wrapper(Q, K, V, t_Q, t_K, t_V, scale: Optional[float] = None,
+                                                 y=None, t_y=None, M=None, MU=None, LI=None,
+                                                 return_M: bool = False):
+    """Signature of ``flash_attention_jvp_multihead_triton_kernel_wrapper`` (ryu_triton.py:295-309):
+    [B,H,L,D] tensors with arbitrary batch/head/sequence strides; returns ``(y, t_y)`` or, with
+    ``return_M``, ``(y, t_y, M, MU, LI)``."""
+    y, t_y, M, MU, LI = attention_jvp_forward(Q, K, V, t_Q, t_K, t_V, scale=scale, o=y, to=t_y,
+                                              lse=M, mu=MU, li=LI)
+    return (y, t_y, M, MU, LI) if return_M else (y, t_y)
+
+
+def _bshd(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return None if t is None else t.transpose(1, 2)
+
+
+def flash_jvp_backward(dto, q, k, v, o, tq, tk, tv, lse, mu, li, dq, dk, dv, dtq, dtk, dtv,
+                       softmax_scale: Optional[float] = None, *, to=None) -> None:
+    """Signature of ``flash_jvp_backward._flash_attn_backward`` (flash_jvp_backward.py:2293-2312):
+    every tensor is [B,S,H,D]; fills the six gradients in place for the cotangent ``dto`` on the
+    tangent output.  ``o`` must be the primal output and ``to`` the tangent output of the forward:
+    the row sums are taken from them instead of being recomputed with five contractions.  ``li`` is
+    accepted and ignored (it is not needed mathematically)."""
+    if to is None:
+        raise ValueError("flash_jvp_backward needs the forward's tangent output as keyword `to` "
+                         "(and its primal output as `o`)")
+    for tan, tan_grad in zip((tq, tk, tv), (dtq, dtk, dtv)):  # flash_jvp_backward.py:2419-2428
+        for i in range(tan.dim()):
+            if tan.shape[i] != tan_grad.shape[i]:
+                raise ValueError(f"Tangent and tangent gradient have different shapes: "
+                                 f"{tan.shape} != {tan_grad.shape}")
+    attention_jvp_backward(_bshd(q), _bshd(k), _bshd(v), _bshd(tq), _bshd(tk), _bshd(tv), _bshd(o),
+                           _bshd(to), lse, mu, dO=None, dTO=_bshd(dto), scale=softmax_scale,
+                           grads=tuple(_bshd(g) for g in (dq, dk, dv, dtq, dtk, dtv)))
+
+
+def flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal: bool = False,
+                        softmax_scale: Optional[float] = None) -> None:
+    """Signature of ``flash_attn_triton._flash_attn_backward`` (flash_attn_triton.py:974-976) as
+    semicat calls it (functional.py:192-205: no bias, non-causal): [B,S,H,D] tensors, fills
+    dq, dk, dv in place for the cotangent ``do`` on the primal output."""
+    if bias is not None or causal:
+        raise NotImplementedError("the attention-JVP path is non-causal and bias-free")
+    attention_jvp_backward(_bshd(q), _bshd(k), _bshd(v), None, None, None, _bshd(o), None, lse, None,
+                           dO=_bshd(do), dTO=None, scale=softmax_scale,
+                           grads=(_bshd(dq), _bshd(dk), _bshd(dv), None, None, None))
+
+
+def default_scale(D: int) -> float:
+    return 1.0 / math.sqrt(D)

@@ -1,0 +1,179 @@
+"""CPU tests of the host side: the autograd wiring of sdpa_jvp / safe_sdpa_jvp (with the kernel
+launchers replaced by eager stand-ins from tests/eager_backend.py), argument checking, and the C-ABI
+library's exported symbols.  No HIP compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import semicat_amd
+from semicat_amd import _lib, build, functional, kernels
+from oracle import attn_jvp_oracle as orc
+
+from . import eager_backend
+
+GRADS = ("dq", "dk", "dv", "dtq", "dtk", "dtv")
+
+
+def _leaf(x, dtype):
+    return x.to(dtype).clone().requires_grad_(True)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_jvp_then_backward_both_cotangents(monkeypatch, dtype, tol):
+    """torch.func.jvp(sdpa_jvp) then reverse mode through BOTH outputs reaches all six inputs and
+    equals the oracle's autograd path (drop-in contract of functional.py:298-301)."""
+    eager_backend.install(monkeypatch)
+    x = orc.make_inputs(2, 2, 24, 40, 16, seed=1, dtype=dtype)
+    leaves = [_leaf(x[n], dtype) for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(functional.sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+    assert y.shape == (2, 2, 24, 16) and y.is_contiguous() and ty.shape == y.shape
+    (y.float() * x["dO"].float()).sum().add((ty.float() * x["dTO"].float()).sum()).backward()
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    assert orc.rel_frobenius(y, ref["O"]) < tol and orc.rel_frobenius(ty, ref["TO"]) < tol
+    for n, leaf in zip(GRADS, leaves):
+        assert leaf.grad is not None, n
+        assert orc.rel_frobenius(leaf.grad, ref[n]) < tol, n
+
+
+@pytest.mark.parametrize("which", ["primal", "tangent"])
+def test_single_cotangent(monkeypatch, which):
+    """Only one of the two autograd nodes receives a cotangent (set_materialize_grads(False),
+    functional.py:237,263-264)."""
+    eager_backend.install(monkeypatch)
+    x = orc.make_inputs(1, 2, 16, 16, 16, seed=2)
+    leaves = [_leaf(x[n], torch.float32) for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(functional.sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+    if which == "primal":
+        (y * x["dO"]).sum().backward()
+        ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], dO=x["dO"])
+        for leaf in leaves[3:]:
+            assert leaf.grad is None
+        names = GRADS[:3]
+    else:
+        (ty * x["dTO"]).sum().backward()
+        ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], dTO=x["dTO"])
+        names = GRADS
+    for n, leaf in zip(names, leaves):
+        assert orc.rel_frobenius(leaf.grad, ref[n]) < 2e-5, n
+
+
+def test_plain_forward_and_backward_without_tangents(monkeypatch):
+    """Without forward-mode tangents the op is ordinary attention (the reference returns garbage
+    here, functional.py:286-287)."""
+    eager_backend.install(monkeypatch)
+    x = orc.make_inputs(1, 2, 16, 24, 16, seed=3)
+    q, k, v = (_leaf(x[n], torch.float32) for n in "qkv")
+    y = functional.sdpa_jvp(q, k, v)
+    (y * x["dO"]).sum().backward()
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], dO=x["dO"])
+    assert orc.rel_frobenius(y, ref["O"]) < 2e-5
+    for n, leaf in zip(GRADS[:3], (q, k, v)):
+        assert orc.rel_frobenius(leaf.grad, ref[n]) < 2e-5, n
+
+
+def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
+    """[B,S,H,D] in and out, fp32 inputs are computed in bf16 and cast back (functional.py:318-332);
+    inside the op q,k,v are [B,H,S,D] views with strides (S*H*D, D, H*D, 1)."""
+    seen = {}
+    real = eager_backend.attention_jvp_forward
+
+    def spy(q, k, v, *a, **kw):
+        seen["strides"] = q.stride()
+        seen["dtype"] = q.dtype
+        return real(q, k, v, *a, **kw)
+
+    eager_backend.install(monkeypatch)
+    monkeypatch.setattr(kernels, "attention_jvp_forward", spy)
+    B, S, H, D = 2, 8, 3, 16
+    g = torch.Generator().manual_seed(0)
+    q, k, v, tq, tk, tv = (torch.randn(B, S, H, D, generator=g) for _ in range(6))
+    y, ty = torch.func.jvp(functional.safe_sdpa_jvp, (q, k, v), (tq, tk, tv))
+    assert y.shape == (B, S, H, D) and y.dtype == torch.float32 and ty.dtype == torch.float32
+    assert seen["strides"] == (S * H * D, D, H * D, 1) and seen["dtype"] == torch.bfloat16
+    ref = orc.attention_jvp_autograd(*(t.transpose(1, 2) for t in (q, k, v, tq, tk, tv)))
+    assert orc.rel_frobenius(y.transpose(1, 2), ref["O"]) < 3e-2
+    assert orc.rel_frobenius(ty.transpose(1, 2), ref["TO"]) < 3e-2
+
+
+def test_through_a_module_with_scalar_time_tangent(monkeypatch):
+    """The training pattern (semicat.py:153-157): jvp w.r.t. a scalar time through a block that
+    modulates the attention input, then backward to the block's weights."""
+    eager_backend.install(monkeypatch)
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(16, 48)
+    x = torch.randn(2, 8, 16)
+
+    def net(t):
+        h = lin(x * (1 + t))
+        q, k, v = h.view(2, 8, 3, 2, 8).permute(2, 0, 1, 3, 4).unbind(0)  # [B,S,H,D] each... D=8 -> pad
+        q, k, v = (torch.cat([z, z], -1) for z in (q, k, v))              # D = 16
+        return functional.safe_sdpa_jvp(q.contiguous(), k.contiguous(), v.contiguous())
+
+    t = torch.tensor(0.3)
+    y, ty = torch.func.jvp(net, (t,), (torch.ones(()),))
+    (y.sum() + (ty ** 2).sum()).backward()
+    assert lin.weight.grad is not None and torch.isfinite(lin.weight.grad).all()
+    assert lin.weight.grad.abs().sum() > 0
+
+
+def test_launchers_refuse_cpu_tensors():
+    """No CPU fallback: the real launchers raise on non-GPU tensors."""
+    q = torch.zeros(1, 1, 8, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.attention_jvp_forward(q, q, q, q, q, q)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.attention_forward(q, q, q)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.attention_jvp_backward(q, q, q, q, q, q, q, q, None, None, dTO=q)
+
+
+def test_library_exports_every_declared_symbol(repo_root):
+    """libsjvp.so loads and exports exactly what include/sjvp.h declares; the functions that need
+    no GPU answer."""
+    header = open(os.path.join(repo_root, "include", "sjvp.h")).read()
+    declared = set(re.findall(r"\b(sjvp_[a-z_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS)
+    if not os.path.exists(build.LIB_PATH):
+        build.build()
+    lib = ctypes.CDLL(build.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    L = _lib.load()
+    assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
+    assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 2 * 64 * 12 * 128 * 4
+    assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 2 * 256 * 4
+    for code in range(0, -8, -1):
+        assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_c_abi_argument_errors_are_reported_before_any_launch():
+    """Argument validation happens on the host before any HIP call, so it can be exercised
+    without a GPU: bad head dims, dtype, shapes, NULLs, missing cotangents, small workspace."""
+    L = _lib.load()
+    strides = (ctypes.c_int64 * 48)(*([0] * 48))
+    one = ctypes.c_void_p(16)  # non-NULL placeholder; never dereferenced on these paths
+    f = lambda **kw: L.sjvp_fwd(one, one, one, one, one, one, one, one, one, one, one,
+                                kw.get("B", 1), 1, kw.get("Lq", 8), 8, kw.get("D", 64), strides, 0.0,
+                                kw.get("dtype", 0), None)
+    assert f(D=8) == _lib.SJVP_ERR_HEAD_DIM       # ryu_triton.py:319-322
+    assert f(D=256) == _lib.SJVP_ERR_HEAD_DIM     # flash_jvp_backward.py:2318
+    assert f(dtype=7) == _lib.SJVP_ERR_DTYPE
+    assert f(B=0) == _lib.SJVP_ERR_SHAPE
+    assert f(Lq=0) == _lib.SJVP_ERR_SHAPE
+    assert L.sjvp_fwd(None, one, one, one, one, one, one, one, one, one, one, 1, 1, 8, 8, 64, strides,
+                      0.0, 0, None) == _lib.SJVP_ERR_NULL
+    # tangent inputs must come all together
+    assert L.sjvp_fwd(one, one, one, one, None, one, one, one, one, one, one, 1, 1, 8, 8, 64, strides,
+                      0.0, 0, None) == _lib.SJVP_ERR_NULL
+    b = lambda dO, dTO, ws, nbytes: L.sjvp_bwd(one, one, one, one, one, one, one, one, dO, dTO, one,
+                                              one, one, one, one, one, one, one, ws, nbytes, 1, 1, 8,
+                                              8, 64, strides, 0.0, 0, None)
+    assert b(None, None, one, 1 << 20) == _lib.SJVP_ERR_COTANGENT
+    assert b(one, one, None, 1 << 20) == _lib.SJVP_ERR_WORKSPACE
+    assert b(one, one, one, 8) == _lib.SJVP_ERR_WORKSPACE
+    with pytest.raises(_lib.SjvpError):
+        _lib.check(_lib.SJVP_ERR_HEAD_DIM)

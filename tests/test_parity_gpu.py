@@ -1,0 +1,270 @@
+"""GPU parity tests: the HIP kernels (called through the C ABI in libsjvp.so) against the fp64
+oracle on the same seeded inputs.  Gate (relative Frobenius error of each of the eight outputs):
+<= 1e-2 for bf16 / fp16 kernels; statistics are fp32 and held to tighter bounds."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_jvp_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL_16BIT = 1e-2
+GRADS = ("dq", "dk", "dv", "dtq", "dtk", "dtv")
+OUTS = ("O", "TO") + GRADS
+# the reference's own test shapes (ryu_triton.py:504-510), fp16, seed 42, tangents * 0.1
+REF_SHAPES = [(1, 1, 8, 16), (2, 2, 16, 32), (1, 4, 32, 32), (1, 1, 64, 64), (2, 3, 128, 16)]
+
+
+@pytest.fixture(scope="module")
+def K():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import semicat_amd.kernels as kernels
+    from semicat_amd import _lib
+    _lib.load()  # fail loudly if the HIP library is missing
+    return kernels
+
+
+def _dev(x):
+    return {n: t.cuda() for n, t in x.items()}
+
+
+def run_hip(K, x, dO=True, dTO=True):
+    """forward + fused backward through the C ABI; everything returned on the CPU."""
+    d = _dev(x)
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"] if dO else None, dTO=d["dTO"] if dTO else None)
+    torch.cuda.synchronize()
+    res = {"O": o, "TO": to, "lse": lse, "mu": mu, "li": li}
+    res.update({n: t for n, t in zip(GRADS, g) if t is not None})
+    return {n: t.cpu() for n, t in res.items()}
+
+
+def errors(res, ref, names=OUTS):
+    return {n: orc.rel_frobenius(res[n], ref[n]) for n in names if n in res}
+
+
+def assert_parity(res, ref, tol, names=OUTS, label=""):
+    err = errors(res, ref, names)
+    print(f"[parity {label}] " + " ".join(f"{n}={e:.2e}" for n, e in err.items()), flush=True)
+    bad = {n: e for n, e in err.items() if not (e <= tol)}
+    assert not bad, f"{label}: relative Frobenius error above {tol}: {bad}"
+    return err
+
+
+def check_stats(res, x, Lq, Lk):
+    cf = orc.attention_jvp_closed_form(*[x[n] for n in orc.TENSOR_ORDER[:6]])
+    np.testing.assert_allclose(res["lse"][..., :Lq].numpy(), cf["lse"], rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(res["li"][..., :Lq].numpy(), cf["li"], rtol=1e-4)
+    scale = np.abs(cf["mu"]).max() + 1e-6
+    assert np.abs(res["mu"][..., :Lq].numpy() - cf["mu"]).max() <= 1e-2 * scale
+    # rows >= Lq hold log(Lk), 0, Lk (functional.py:57-59,228-229)
+    if res["lse"].shape[-1] > Lq:
+        np.testing.assert_allclose(res["lse"][..., Lq:].numpy(), math.log(Lk), rtol=1e-6)
+        assert (res["mu"][..., Lq:] == 0).all()
+        assert (res["li"][..., Lq:] == Lk).all()
+
+
+@pytest.mark.parametrize("shape", REF_SHAPES)
+def test_reference_test_shapes_fp16(K, shape):
+    """The reference's forward test (ryu_triton.py:495-592) on its shapes, extended to the backward."""
+    B, H, L, D = shape
+    x = orc.make_inputs(B, H, L, L, D, seed=42, tangent_scale=0.1, dtype=torch.float16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    assert_parity(res, ref, TOL_16BIT, label=f"fp16 {shape}")
+    # the authors' own criterion: rtol = atol = 1e-2 on y and t_y (ryu_triton.py:551-554)
+    assert torch.allclose(res["O"].double(), ref["O"], rtol=1e-2, atol=1e-2)
+    assert torch.allclose(res["TO"].double(), ref["TO"], rtol=1e-2, atol=1e-2)
+    check_stats(res, x, L, L)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Lq,Lk,D", [
+    (2, 3, 128, 128, 64),    # one full block, the metric's tile shape
+    (1, 2, 256, 256, 64),    # two blocks each way
+    (2, 2, 100, 77, 64),     # ragged both ways
+    (1, 2, 33, 200, 32),     # Lq != Lk, several key stages
+    (1, 1, 300, 41, 16),     # several query blocks, ragged keys inside the first tile pair
+    (1, 2, 130, 130, 128),   # D = 128
+    (1, 1, 64, 96, 48),      # D not a power of two
+    (1, 1, 1, 1, 16),        # degenerate
+])
+def test_forward_backward_parity(K, dtype, B, H, Lq, Lk, D):
+    x = orc.make_inputs(B, H, Lq, Lk, D, seed=0, dtype=dtype)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    assert_parity(res, ref, TOL_16BIT, label=f"{dtype} {(B, H, Lq, Lk, D)}")
+    check_stats(res, x, Lq, Lk)
+
+
+@pytest.mark.parametrize("which", ["dO", "dTO"])
+@pytest.mark.parametrize("B,H,Lq,Lk,D", [(2, 2, 128, 128, 64), (1, 2, 70, 150, 32), (1, 1, 40, 40, 128)])
+def test_single_cotangent_modes(K, which, B, H, Lq, Lk, D):
+    """Each autograd node calls the backward with one cotangent (functional.py:72-87, 261-268)."""
+    x = orc.make_inputs(B, H, Lq, Lk, D, seed=3, dtype=torch.bfloat16)
+    a = [x[n] for n in orc.TENSOR_ORDER[:6]]
+    if which == "dO":
+        ref = orc.attention_jvp_autograd(*a, dO=x["dO"])
+        res = run_hip(K, x, dO=True, dTO=False)
+        assert "dtq" not in res
+        assert_parity(res, ref, TOL_16BIT, names=("dq", "dk", "dv"), label=f"dO-only {(B, H, Lq, Lk, D)}")
+    else:
+        ref = orc.attention_jvp_autograd(*a, dTO=x["dTO"])
+        res = run_hip(K, x, dO=False, dTO=True)
+        assert_parity(res, ref, TOL_16BIT, names=GRADS, label=f"dTO-only {(B, H, Lq, Lk, D)}")
+
+
+def test_primal_only_forward(K):
+    x = orc.make_inputs(2, 2, 150, 90, 64, seed=4, dtype=torch.bfloat16)
+    d = _dev(x)
+    o, lse = K.attention_forward(d["q"], d["k"], d["v"])
+    cf = orc.attention_jvp_closed_form(*[x[n] for n in orc.TENSOR_ORDER[:6]])
+    assert orc.rel_frobenius(o.cpu(), cf["O"]) <= TOL_16BIT
+    np.testing.assert_allclose(lse[..., :150].cpu().numpy(), cf["lse"], rtol=2e-5, atol=2e-5)
+
+
+def test_caller_layout_strided_views(K):
+    """duo.py:141 hands [B,S,H,D]-contiguous tensors; inside the op they are [B,H,S,D] views with
+    strides (S*H*D, D, H*D, 1).  Gradients come back with the strides of their inputs."""
+    B, H, L, D = 2, 3, 96, 64
+    x = orc.make_inputs(B, H, L, L, D, seed=5, dtype=torch.bfloat16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    d = {n: t.cuda().transpose(1, 2).contiguous().transpose(1, 2) for n, t in x.items()}
+    assert d["q"].stride() == (L * H * D, D, H * D, 1)
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    assert o.is_contiguous() and to.is_contiguous()
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    for t in g:
+        assert t.stride() == (L * H * D, D, H * D, 1)
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g)}}
+    assert_parity(res, ref, TOL_16BIT, label="strided")
+
+
+def test_unaligned_and_odd_head_dim_take_the_scalar_path(K):
+    """D = 20 (not a multiple of 8) and a base pointer offset by one element."""
+    B, H, L, D = 1, 2, 50, 20
+    x = orc.make_inputs(B, H, L, L, D, seed=6, dtype=torch.float16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    assert_parity(res, ref, TOL_16BIT, label="D=20")
+    D = 32
+    x = orc.make_inputs(B, H, L, L, D, seed=6, dtype=torch.float16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    d = {}
+    for n, t in x.items():
+        buf = torch.zeros(t.numel() + 1, dtype=t.dtype, device="cuda")
+        d[n] = buf[1:].view(t.shape).copy_(t.cuda())
+        assert d[n].data_ptr() % 16 != 0
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g)}}
+    assert_parity(res, ref, TOL_16BIT, label="misaligned")
+
+
+def test_bitwise_determinism(K):
+    x = orc.make_inputs(2, 2, 200, 136, 64, seed=7, dtype=torch.bfloat16)
+    a = run_hip(K, x)
+    b = run_hip(K, x)
+    for n in a:
+        assert torch.equal(a[n], b[n]), n
+
+
+def test_metric_config_full_size_against_oracle(K):
+    """Config 2 (B=64,H=12,L=128,D=64, bf16, primal*0.5, tangent*0.1, seed 0) at its full size against
+    the fp64 oracle, and against the emulated error of the reference's own rounding points."""
+    x = orc.make_inputs(64, 12, 128, 128, 64, seed=0, primal_scale=0.5, tangent_scale=0.1,
+                        dtype=torch.bfloat16)
+    a = [x[n] for n in orc.TENSOR_ORDER]
+    ref = orc.attention_jvp_closed_form(*a)
+    res = run_hip(K, x)
+    err = assert_parity(res, ref, TOL_16BIT, label="config 2")
+    sub = {n: t[:4] for n, t in x.items()}
+    model = orc.reference_rounding_error_model(*[sub[n] for n in orc.TENSOR_ORDER])
+    ref_sub = {n: ref[n][:4] for n in OUTS}
+    model_err = errors(model, ref_sub)
+    print("[reference rounding model] " + " ".join(f"{n}={e:.2e}" for n, e in model_err.items()),
+          flush=True)
+    for n in OUTS:
+        assert err[n] <= 1.25 * model_err[n] + 5e-4, (n, err[n], model_err[n])
+
+
+@pytest.mark.parametrize("B,H,L,D,ps,ts", [(128, 12, 256, 64, 1.0, 1.0), (8, 16, 2048, 64, 1.0, 0.1),
+                                           (8, 16, 1024, 128, 1.0, 0.1)])
+def test_large_configs_on_head_slices_and_properties(K, B, H, L, D, ps, ts):
+    """Configs 3 and 4 at full size: (b,h) pairs are independent problems, so a handful of them is
+    checked against the fp64 oracle exactly; the whole output is checked through linearity in the
+    tangents (TO(2*t) = 2*TO(t), O unchanged) and finiteness."""
+    x = orc.make_inputs(B, H, L, L, D, seed=0, primal_scale=ps, tangent_scale=ts, dtype=torch.bfloat16)
+    d = _dev(x)
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    o2, to2, _, _, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], 2 * d["tq"], 2 * d["tk"],
+                                               2 * d["tv"])
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2)
+    assert orc.rel_frobenius(to2.float().cpu(), 2 * to.float().cpu()) < 4e-3
+    for t in (o, to) + tuple(g):
+        assert torch.isfinite(t).all()
+    rng = np.random.default_rng(0)
+    for _ in range(3):
+        b, h = int(rng.integers(B)), int(rng.integers(H))
+        sl = {n: t[b:b + 1, h:h + 1] for n, t in x.items()}
+        ref = orc.attention_jvp_closed_form(*[sl[n] for n in orc.TENSOR_ORDER])
+        res = {"O": o, "TO": to, **dict(zip(GRADS, g))}
+        res = {n: t[b:b + 1, h:h + 1].cpu() for n, t in res.items()}
+        assert_parity(res, ref, TOL_16BIT, label=f"slice ({b},{h}) of {(B, H, L, D)}")
+
+
+def test_autograd_end_to_end_on_gpu(K):
+    """torch.func.jvp(sdpa_jvp) then backward through both outputs, all on the HIP kernels."""
+    from semicat_amd import sdpa_jvp, safe_sdpa_jvp
+    B, H, L, D = 2, 4, 128, 64
+    x = orc.make_inputs(B, H, L, L, D, seed=8, tangent_scale=0.1, dtype=torch.bfloat16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    leaves = [x[n].cuda().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+    loss = (y.float() * x["dO"].cuda().float()).sum() + (ty.float() * x["dTO"].cuda().float()).sum()
+    loss.backward()
+    res = {"O": y.detach().cpu(), "TO": ty.detach().cpu(),
+           **{n: l.grad.cpu() for n, l in zip(GRADS, leaves)}}
+    # dq, dk, dv are the 16-bit sum of two separately rounded launches here
+    assert_parity(res, ref, 1.2e-2, label="autograd")
+    # plain call (no tangents) computes attention; [B,S,H,D] fp32 wrapper casts and transposes
+    q32 = x["q"].float().cuda().transpose(1, 2).contiguous()
+    k32 = x["k"].float().cuda().transpose(1, 2).contiguous()
+    v32 = x["v"].float().cuda().transpose(1, 2).contiguous()
+    y2 = safe_sdpa_jvp(q32, k32, v32)
+    assert y2.dtype == torch.float32 and y2.shape == (B, L, H, D)
+    assert orc.rel_frobenius(y2.transpose(1, 2).cpu(), ref["O"]) <= TOL_16BIT
+
+
+def test_reference_signature_wrappers(K):
+    """The three drop-in launchers with the reference's own argument lists and layouts."""
+    B, H, L, D = 2, 2, 64, 32
+    x = orc.make_inputs(B, H, L, L, D, seed=9, dtype=torch.float16)
+    ref_g = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], dTO=x["dTO"])
+    ref_p = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], dO=x["dO"])
+    d = _dev(x)
+    y, t_y, M, MU, LI = K.flash_attention_jvp_multihead_kernel_wrapper(
+        d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], return_M=True)
+    assert M.shape == (B, H, 128)
+    f = lambda t: t.transpose(1, 2)  # [B,H,S,D] -> the [B,S,H,D] views the reference passes
+    grads = [torch.empty_like(f(d[n])) for n in ("q", "k", "v", "tq", "tk", "tv")]
+    K.flash_jvp_backward(f(d["dTO"]), f(d["q"]), f(d["k"]), f(d["v"]), f(y), f(d["tq"]), f(d["tk"]),
+                         f(d["tv"]), M, MU, LI, *grads, to=f(t_y))
+    res = {n: g.transpose(1, 2).cpu() for n, g in zip(GRADS, grads)}
+    assert_parity(res, ref_g, TOL_16BIT, names=GRADS, label="flash_jvp_backward")
+    dq, dk, dv = (torch.empty_like(f(d[n])) for n in "qkv")
+    K.flash_attn_backward(f(d["dO"]), f(d["q"]), f(d["k"]), f(d["v"]), f(y), M, dq, dk, dv)
+    res = {n: g.transpose(1, 2).cpu() for n, g in zip(("dq", "dk", "dv"), (dq, dk, dv))}
+    assert_parity(res, ref_p, TOL_16BIT, names=("dq", "dk", "dv"), label="flash_attn_backward")
+    with pytest.raises(ValueError):
+        K.flash_attention_jvp_multihead_kernel_wrapper(*(d[n][..., :8] for n in
+                                                         ("q", "k", "v", "tq", "tk", "tv")))
