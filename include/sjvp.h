@@ -86,7 +86,8 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
              void* dtv, void* workspace, size_t workspace_bytes, int B, int H, int Lq, int Lk, int D,
              const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
 
-/* Bytes of caller-provided device scratch sjvp_bwd needs (row sums sum_4 and sum_7 + delta, which
+/* Bytes of caller-provided device scratch sjvp_bwd needs (lse in log2 units and the row sums sum_4 and
+ * sum_7 + delta, which
  * the reference allocates itself at flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
 

@@ -54,59 +54,88 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
     return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
 }
 
-template <typename T, int HD>
+// Ring depth (stages of 32 rows in flight) per head-dimension class.
+template <int HD>
+struct Ring {
+    static constexpr int depth = HD == 128 ? 3 : 4;
+};
+
+template <typename T, int HD, bool DMA>
 int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    constexpr int BN = 64;
-    if (jvp) return launch(fwd_kernel<T, HD, BN, true>, grid, FwdSmem<HD, BN, true>::bytes, stream, p);
-    return launch(fwd_kernel<T, HD, BN, false>, grid, FwdSmem<HD, BN, false>::bytes, stream, p);
+    constexpr int R = DMA ? Ring<HD>::depth : 1;
+    if (jvp)
+        return launch(fwd_kernel<T, HD, R, true, DMA>, grid, FwdSmem<HD, R, true>::bytes, stream, p);
+    return launch(fwd_kernel<T, HD, R, false, DMA>, grid, FwdSmem<HD, R, false>::bytes, stream, p);
 }
 
 template <typename T>
 int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    if (p.D <= 32) return fwd_hd<T, 32>(p, grid, jvp, stream);
-    if (p.D <= 64) return fwd_hd<T, 64>(p, grid, jvp, stream);
-    return fwd_hd<T, 128>(p, grid, jvp, stream);
+    // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
+    if (p.vec) {
+        if (p.D <= 32) return fwd_hd<T, 32, true>(p, grid, jvp, stream);
+        if (p.D <= 64) return fwd_hd<T, 64, true>(p, grid, jvp, stream);
+        return fwd_hd<T, 128, true>(p, grid, jvp, stream);
+    }
+    if (p.D <= 32) return fwd_hd<T, 32, false>(p, grid, jvp, stream);
+    if (p.D <= 64) return fwd_hd<T, 64, false>(p, grid, jvp, stream);
+    return fwd_hd<T, 128, false>(p, grid, jvp, stream);
 }
 
-template <typename T, int HD, bool HAS_DO, bool HAS_G>
+template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
 int bwd_mode(const BwdParams& p, int BH, hipStream_t stream) {
-    int rc = launch(bwd_rowstats_kernel<T, HAS_DO, HAS_G>, BH * (p.Lr / 32), 0, stream, p);
+    constexpr int R = DMA ? Ring<HD>::depth : 1;
+    // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.
+    int rc = launch(bwd_row_kernel<T, HD, R, HAS_DO, HAS_G, DMA>, BH * p.q_blocks,
+                    RowSmem<HD, R, HAS_G>::bytes, stream, p);
     if (rc != SJVP_OK) return rc;
     const int col_grid = BH * p.k_blocks;
+    using SM = ColSmem<HD, R, HAS_DO, HAS_G>;
     if constexpr (HD == 128) {
         // two launches, each accumulating half of the head dimension (register budget)
-        constexpr int BM = 32;
-        using SM = ColSmem<HD, BM, HAS_DO, HAS_G>;
-        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 0, 2>, col_grid, SM::bytes, stream, p);
+        rc = launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 0, 2, DMA>, col_grid, SM::bytes,
+                    stream, p);
         if (rc != SJVP_OK) return rc;
-        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 2, 2>, col_grid, SM::bytes, stream, p);
+        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 2, 2, DMA>, col_grid,
+                      SM::bytes, stream, p);
     } else {
-        constexpr int BM = 64;
-        using SM = ColSmem<HD, BM, HAS_DO, HAS_G>;
-        rc = launch(bwd_col_kernel<T, HD, BM, HAS_DO, HAS_G, 0, HD / 32>, col_grid, SM::bytes, stream,
-                    p);
+#ifdef SJVP_X_SPLITCOL
+        rc = launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, false, 0, HD / 32, DMA>, col_grid,
+                    SM::bytes, stream, p);
+        if (rc != SJVP_OK) return rc;
+        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, false, true, 0, HD / 32, DMA>, col_grid,
+                      SM::bytes, stream, p);
+#else
+        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 0, HD / 32, DMA>, col_grid,
+                      SM::bytes, stream, p);
+#endif
     }
-    if (rc != SJVP_OK) return rc;
-    constexpr int BN = 64;
-    return launch(bwd_row_kernel<T, HD, BN, HAS_DO, HAS_G>, BH * p.q_blocks,
-                  RowSmem<HD, BN, HAS_G>::bytes, stream, p);
 }
 
-template <typename T, int HD>
+template <typename T, int HD, bool DMA>
 int bwd_hd(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
-    if (has_do && has_g) return bwd_mode<T, HD, true, true>(p, BH, stream);
-    if (has_g) return bwd_mode<T, HD, false, true>(p, BH, stream);
-    return bwd_mode<T, HD, true, false>(p, BH, stream);
+    if (has_do && has_g) return bwd_mode<T, HD, true, true, DMA>(p, BH, stream);
+    if (has_g) return bwd_mode<T, HD, false, true, DMA>(p, BH, stream);
+    return bwd_mode<T, HD, true, false, DMA>(p, BH, stream);
 }
 
 template <typename T>
 int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
-    if (p.D <= 32) return bwd_hd<T, 32>(p, BH, has_do, has_g, stream);
-    if (p.D <= 64) return bwd_hd<T, 64>(p, BH, has_do, has_g, stream);
-    return bwd_hd<T, 128>(p, BH, has_do, has_g, stream);
+    if (p.vec) {
+        if (p.D <= 32) return bwd_hd<T, 32, true>(p, BH, has_do, has_g, stream);
+        if (p.D <= 64) return bwd_hd<T, 64, true>(p, BH, has_do, has_g, stream);
+        return bwd_hd<T, 128, true>(p, BH, has_do, has_g, stream);
+    }
+    if (p.D <= 32) return bwd_hd<T, 32, false>(p, BH, has_do, has_g, stream);
+    if (p.D <= 64) return bwd_hd<T, 64, false>(p, BH, has_do, has_g, stream);
+    return bwd_hd<T, 128, false>(p, BH, has_do, has_g, stream);
 }
 
 }  // namespace
+
+#ifdef SJVP_X_TIMING
+static unsigned long long* g_dbg = nullptr;
+extern "C" void sjvp_x_set_debug(void* p) { g_dbg = static_cast<unsigned long long*>(p); }
+#endif
 
 extern "C" {
 
@@ -131,15 +160,9 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
         p.tq = view(tq, strides + 3 * SJVP_F_TQ);
         p.tk = view(tk, strides + 3 * SJVP_F_TK);
         p.tv = view(tv, strides + 3 * SJVP_F_TV);
-        p.to = static_cast<elem_t*>(to);
-        p.to_sb = strides[3 * SJVP_F_TO];
-        p.to_sh = strides[3 * SJVP_F_TO + 1];
-        p.to_sl = strides[3 * SJVP_F_TO + 2];
+        p.to = out_view(to, strides + 3 * SJVP_F_TO);
     }
-    p.o = static_cast<elem_t*>(o);
-    p.o_sb = strides[3 * SJVP_F_O];
-    p.o_sh = strides[3 * SJVP_F_O + 1];
-    p.o_sl = strides[3 * SJVP_F_O + 2];
+    p.o = out_view(o, strides + 3 * SJVP_F_O);
     p.lse = lse;
     p.mu = mu;
     p.li = li;
@@ -152,6 +175,9 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
+#ifdef SJVP_X_TIMING
+    p.dbg = g_dbg;
+#endif
     const int grid = B * H * p.q_blocks;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == SJVP_BF16 ? fwd_dtype<Bf16>(p, grid, jvp, s) : fwd_dtype<Fp16>(p, grid, jvp, s);
@@ -162,7 +188,7 @@ size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype) 
     (void)D;
     (void)dtype;
     if (B < 1 || H < 1 || Lq < 1) return 0;
-    return (size_t)2 * (size_t)B * (size_t)H * (size_t)round_up(Lq, 128) * sizeof(float);
+    return (size_t)3 * (size_t)B * (size_t)H * (size_t)round_up(Lq, 128) * sizeof(float);
 }
 
 int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
@@ -215,11 +241,15 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.Lr = round_up(Lq, 128);
     p.q_blocks = p.Lr / 128;
     p.k_blocks = round_up(Lk, 128) / 128;
-    p.s4 = static_cast<float*>(workspace);
+    p.lse2 = static_cast<float*>(workspace);
+    p.s4 = p.lse2 + (size_t)B * H * p.Lr;
     p.s7d = p.s4 + (size_t)B * H * p.Lr;
     p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
+#ifdef SJVP_X_TIMING
+    p.dbg = g_dbg;
+#endif
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, s)
                               : bwd_dtype<Fp16>(p, B * H, has_do, has_g, s);

@@ -10,304 +10,59 @@
 //     dV_dot = P^T G            dV = P_dot^T G + P^T dO
 //     dK_dot = s dS_dot^T Q     dK = s (dS^T Q + dS_dot^T Q_dot)
 //     dQ_dot = s dS_dot K       dQ = s (dS K + dS_dot K_dot)
-// The reference spends eight launches and 35 tile contractions on this; here it is three launches:
-//   bwd_rowstats_kernel  s4, s7d from O, TO, dO, G (O(L*D) work instead of five contractions),
-//   bwd_col_kernel       a wavefront owns 32 keys  -> dK, dV, dK_dot, dV_dot,
-//   bwd_row_kernel       a wavefront owns 32 queries -> dQ, dQ_dot,
+// The reference spends eight launches and 35 tile contractions on this; here it is two launches:
+//   bwd_row_kernel   a wavefront owns 32 queries -> dQ, dQ_dot; it also forms s4 and s7d for its
+//                    rows from O, TO, dO, G (O(L*D) work instead of five contractions) and leaves
+//                    them, with lse in log2 units, in the workspace for
+//   bwd_col_kernel   a wavefront owns 32 keys  -> dK, dV, dK_dot, dV_dot,
 // each gradient accumulated in fp32 registers by exactly one wavefront and written once, so the
 // result is deterministic and never round-trips through 16-bit partial sums.
 #pragma once
+#include <type_traits>
+
 #include "sjvp_device.hpp"
 
 namespace sjvp {
-
-struct OutView {
-    elem_t* ptr;
-    int64_t sb, sh, sl;
-    __device__ __forceinline__ elem_t* head(int b, int h) const { return ptr + b * sb + h * sh; }
-};
 
 struct BwdParams {
     TensorView q, k, v, tq, tk, tv, o, to, dO, dTO;
     OutView dq, dk, dv, dtq, dtk, dtv;
     const float* lse;
     const float* mu;
-    float* s4;   // [B*H][Lr]  rowsum(G*O)
-    float* s7d;  // [B*H][Lr]  rowsum(G*TO) + rowsum(dO*O)
+    float* lse2;  // workspace [B*H][Lr]  lse * log2(e)
+    float* s4;    // workspace [B*H][Lr]  rowsum(G*O)
+    float* s7d;   // workspace [B*H][Lr]  rowsum(G*TO) + rowsum(dO*O)
     int H, Lq, Lk, D, Lr;
     int q_blocks, k_blocks;  // ceil(L / 128)
     float scale;
     int vec;
+#ifdef SJVP_X_TIMING
+    unsigned long long* dbg;
+#endif
 };
-
-// ---------------------------------------------------------------------------------------------
-// Row sums.  Eight lanes per query row, 32 rows per workgroup.
-template <typename T, bool HAS_DO, bool HAS_G>
-__global__ __launch_bounds__(kThreads) void bwd_rowstats_kernel(const BwdParams p) {
-    const int tid = threadIdx.x;
-    const int sub = tid & 7;
-    const int blocks_per_head = p.Lr / 32;
-    const int bh = blockIdx.x / blocks_per_head;
-    const int row = (blockIdx.x % blocks_per_head) * 32 + (tid >> 3);
-    const int b = bh / p.H, h = bh % p.H;
-    const bool valid = row < p.Lq;
-    const bool vec = p.vec != 0;
-    float a4 = 0.f, a7 = 0.f;
-    if (valid) {
-        const elem_t* orow = p.o.head(b, h) + (int64_t)row * p.o.sl;
-        const elem_t* torow = HAS_G ? p.to.head(b, h) + (int64_t)row * p.to.sl : nullptr;
-        const elem_t* grow = HAS_G ? p.dTO.head(b, h) + (int64_t)row * p.dTO.sl : nullptr;
-        const elem_t* drow = HAS_DO ? p.dO.head(b, h) + (int64_t)row * p.dO.sl : nullptr;
-        for (int d = 8 * sub; d < p.D; d += 64) {
-            u32x4 ov = load8(orow, d, p.D, true, vec);
-            u32x4 tov, gv, dv;
-            if constexpr (HAS_G) {
-                tov = load8(torow, d, p.D, true, vec);
-                gv = load8(grow, d, p.D, true, vec);
-            }
-            if constexpr (HAS_DO) dv = load8(drow, d, p.D, true, vec);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int sh = 16 * (i & 1);
-                float of = T::to_float((elem_t)((ov[i >> 1] >> sh) & 0xffffu));
-                if constexpr (HAS_G) {
-                    float gf = T::to_float((elem_t)((gv[i >> 1] >> sh) & 0xffffu));
-                    float tf = T::to_float((elem_t)((tov[i >> 1] >> sh) & 0xffffu));
-                    a4 += gf * of;
-                    a7 += gf * tf;
-                }
-                if constexpr (HAS_DO) {
-                    float df = T::to_float((elem_t)((dv[i >> 1] >> sh) & 0xffffu));
-                    a7 += df * of;
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 1; m < 8; m <<= 1) {
-        a4 += __shfl_xor(a4, m, 64);
-        a7 += __shfl_xor(a7, m, 64);
-    }
-    if (sub == 0) {
-        p.s4[(int64_t)bh * p.Lr + row] = a4;
-        p.s7d[(int64_t)bh * p.Lr + row] = a7;
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Column-owned kernel: dK, dV (and dK_dot, dV_dot).  Accumulates head-dimension tiles
-// [DT0, DT0 + NDT) only; at HD = 128 it is launched twice to stay inside the register file.
-template <int HD, int BM, bool HAS_DO, bool HAS_G>
-struct ColSmem {
-    static constexpr int tile = BM * Pitch<HD>::value;
-    static constexpr int ntiles = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
-    static constexpr int bytes = ntiles * tile * (int)sizeof(elem_t) + 4 * BM * (int)sizeof(float);
-};
-
-template <typename T, int HD, int BM, bool HAS_DO, bool HAS_G, int DT0, int NDT>
-__global__ __launch_bounds__(kThreads) void bwd_col_kernel(const BwdParams p) {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = ColSmem<HD, BM, HAS_DO, HAS_G>;
-    float* sStat = reinterpret_cast<float*>(smem_raw);  // [4][BM]: lse*log2e, mu, s4, s7d
-    elem_t* sQ = reinterpret_cast<elem_t*>(smem_raw + 4 * BM * sizeof(float));
-    elem_t* sTQ = sQ + SM::tile;                 // HAS_G
-    elem_t* sG = sTQ + SM::tile;                 // HAS_G
-    elem_t* sDO = HAS_G ? sG + SM::tile : sQ + SM::tile;  // HAS_DO
-
-    constexpr int KC = HD / 16;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int x = lane & 31;
-    const int hf = lane >> 5;
-    const int bh = blockIdx.x / p.k_blocks;
-    const int kb = blockIdx.x % p.k_blocks;
-    const int b = bh / p.H, h = bh % p.H;
-    const bool vec = p.vec != 0;
-
-    const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
-    const bool kvalid = krow < p.Lk;
-    const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;
-
-    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    {
-        const elem_t* kp = p.k.head(b, h) + (int64_t)krow * p.k.sl;
-        const elem_t* vp = p.v.head(b, h) + (int64_t)krow * p.v.sl;
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
-            kB[c] = load8(kp, 16 * c + 8 * hf, p.D, kvalid, vec);
-            vB[c] = load8(vp, 16 * c + 8 * hf, p.D, kvalid, vec);
-        }
-        if constexpr (HAS_G) {
-            const elem_t* tkp = p.tk.head(b, h) + (int64_t)krow * p.tk.sl;
-            const elem_t* tvp = p.tv.head(b, h) + (int64_t)krow * p.tv.sl;
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                tkB[c] = load8(tkp, 16 * c + 8 * hf, p.D, kvalid, vec);
-                tvB[c] = load8(tvp, 16 * c + 8 * hf, p.D, kvalid, vec);
-            }
-        }
-    }
-
-    const elem_t* qg = p.q.head(b, h);
-    const elem_t* tqg = HAS_G ? p.tq.head(b, h) : nullptr;
-    const elem_t* gg = HAS_G ? p.dTO.head(b, h) : nullptr;
-    const elem_t* dog = HAS_DO ? p.dO.head(b, h) : nullptr;
-    const float sl2 = p.scale * kLog2e;
-
-    f32x16 dk[NDT], dv[NDT], dtk[NDT], dtv[NDT];
-#pragma unroll
-    for (int t = 0; t < NDT; ++t) {
-        dk[t] = f32x16{0};
-        dv[t] = f32x16{0};
-        if constexpr (HAS_G) {
-            dtk[t] = f32x16{0};
-            dtv[t] = f32x16{0};
-        }
-    }
-
-    for (int q0 = 0; q0 < p.Lq; q0 += BM) {
-        __syncthreads();
-        stage_rows<HD, BM>(sQ, qg, p.q.sl, q0, p.Lq, p.D, vec, tid);
-        if constexpr (HAS_G) {
-            stage_rows<HD, BM>(sTQ, tqg, p.tq.sl, q0, p.Lq, p.D, vec, tid);
-            stage_rows<HD, BM>(sG, gg, p.dTO.sl, q0, p.Lq, p.D, vec, tid);
-        }
-        if constexpr (HAS_DO) stage_rows<HD, BM>(sDO, dog, p.dO.sl, q0, p.Lq, p.D, vec, tid);
-        if (tid < BM) {
-            // Rows beyond Lq are staged as zeros everywhere: their P is finite (= 1) and multiplies
-            // zero rows of Q, Q_dot, G, dO in every contraction below.
-            const int row = q0 + tid;
-            const bool rv = row < p.Lq;
-            const int64_t so = (int64_t)bh * p.Lr + row;
-            sStat[0 * BM + tid] = rv ? p.lse[so] * kLog2e : 0.f;
-            sStat[1 * BM + tid] = (rv && HAS_G) ? p.mu[so] : 0.f;
-            sStat[2 * BM + tid] = rv ? p.s4[so] : 0.f;
-            sStat[3 * BM + tid] = rv ? p.s7d[so] : 0.f;
-        }
-        __syncthreads();
-        if (!wave_active) continue;
-
-#pragma unroll
-        for (int t = 0; t < BM / 32; ++t) {
-            const int y0 = 32 * t;
-            if (q0 + y0 >= p.Lq) break;
-            // tiles: rows = queries (registers), columns = this wave's keys (lanes)
-            f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                u32x4 aq = lds_a_rows<HD>(sQ, y0, c, x, hf);
-                s = T::mfma(aq, kB[c], s);
-                if constexpr (HAS_G) {
-                    ts = T::mfma(aq, tkB[c], ts);
-                    u32x4 atq = lds_a_rows<HD>(sTQ, y0, c, x, hf);
-                    ts = T::mfma(atq, kB[c], ts);
-                    u32x4 ag = lds_a_rows<HD>(sG, y0, c, x, hf);
-                    w = T::mfma(ag, vB[c], w);
-                    xy = T::mfma(ag, tvB[c], xy);
-                }
-                if constexpr (HAS_DO) {
-                    u32x4 ado = lds_a_rows<HD>(sDO, y0, c, x, hf);
-                    xy = T::mfma(ado, vB[c], xy);
-                }
-            }
-            // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const int r0 = y0 + 8 * jj + 4 * hf;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * BM + r0);
-                const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * BM + r0);
-                const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * BM + r0);
-                const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * BM + r0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = 4 * jj + i;
-                    const float pj = fast_exp2(s[j] * sl2 - lse4[i]);
-                    s[j] = pj;
-                    if constexpr (HAS_G) {
-                        const float n = ts[j] * p.scale - mu4[i];
-                        const float dts = pj * (w[j] - s44[i]);
-                        w[j] = dts;
-                        xy[j] = dts * n + pj * (xy[j] - s74[i]);
-                        ts[j] = pj * n;
-                    } else {
-                        xy[j] = pj * (xy[j] - s74[i]);
-                    }
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const u32x4 pB = pack_b<T>(s, c);
-                const u32x4 dsB = pack_b<T>(xy, c);
-                u32x4 pdB, dtsB;
-                if constexpr (HAS_G) {
-                    pdB = pack_b<T>(ts, c);
-                    dtsB = pack_b<T>(w, c);
-                }
-#pragma unroll
-                for (int d = 0; d < NDT; ++d) {
-                    const int d0 = 32 * (DT0 + d);
-                    const u32x4 aq = lds_a_transposed<HD>(sQ, y0, c, d0, lane);
-                    dk[d] = T::mfma(aq, dsB, dk[d]);
-                    if constexpr (HAS_G) {
-                        dtk[d] = T::mfma(aq, dtsB, dtk[d]);
-                        const u32x4 atq = lds_a_transposed<HD>(sTQ, y0, c, d0, lane);
-                        dk[d] = T::mfma(atq, dtsB, dk[d]);
-                        const u32x4 ag = lds_a_transposed<HD>(sG, y0, c, d0, lane);
-                        dtv[d] = T::mfma(ag, pB, dtv[d]);
-                        dv[d] = T::mfma(ag, pdB, dv[d]);
-                    }
-                    if constexpr (HAS_DO) {
-                        const u32x4 ado = lds_a_transposed<HD>(sDO, y0, c, d0, lane);
-                        dv[d] = T::mfma(ado, pB, dv[d]);
-                    }
-                }
-            }
-        }
-    }
-
-    if (!kvalid) return;
-    elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;
-    elem_t* dvrow = p.dv.head(b, h) + (int64_t)krow * p.dv.sl;
-#pragma unroll
-    for (int d = 0; d < NDT; ++d) {
-        store_acc<T>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
-        store_acc<T>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
-    }
-    if constexpr (HAS_G) {
-        elem_t* dtkrow = p.dtk.head(b, h) + (int64_t)krow * p.dtk.sl;
-        elem_t* dtvrow = p.dtv.head(b, h) + (int64_t)krow * p.dtv.sl;
-#pragma unroll
-        for (int d = 0; d < NDT; ++d) {
-            store_acc<T>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
-            store_acc<T>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
-        }
-    }
-}
 
 // ---------------------------------------------------------------------------------------------
 // Row-owned kernel: dQ (and dQ_dot).  Tiles are transposed (rows = keys in registers, columns =
 // this wave's queries in lanes), so the row statistics are per-lane scalars.
-template <int HD, int BN, bool HAS_G>
+template <int HD, int R, bool HAS_G>
 struct RowSmem {
-    static constexpr int tile = BN * Pitch<HD>::value;
-    static constexpr int bytes = (HAS_G ? 4 : 2) * tile * (int)sizeof(elem_t);
+    static constexpr int nt = HAS_G ? 4 : 2;
+    static constexpr int slot = nt * Slab<HD>::elems;
+    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, int BN, bool HAS_DO, bool HAS_G>
-__global__ __launch_bounds__(kThreads) void bwd_row_kernel(const BwdParams p) {
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
+__global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = RowSmem<HD, BN, HAS_G>;
-    elem_t* sK = reinterpret_cast<elem_t*>(smem_raw);
-    elem_t* sV = sK + SM::tile;
-    elem_t* sTK = sV + SM::tile;   // HAS_G
-    elem_t* sTV = sTK + SM::tile;  // HAS_G
+    using SM = RowSmem<HD, R, HAS_G>;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
 
     constexpr int KC = HD / 16;
     constexpr int DT = HD / 32;
+    constexpr int SPT = SM::nt * Slab<HD>::per_thread;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int x = lane & 31;
     const int hf = lane >> 5;
     const int bh = blockIdx.x / p.q_blocks;
@@ -315,6 +70,8 @@ __global__ __launch_bounds__(kThreads) void bwd_row_kernel(const BwdParams p) {
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
 
+    SJVP_TS_DECL;
+    SJVP_TS(0);
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -343,14 +100,76 @@ __global__ __launch_bounds__(kThreads) void bwd_row_kernel(const BwdParams p) {
     const int64_t so = (int64_t)bh * p.Lr + qrow;
     const float lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
     const float mu = (qvalid && HAS_G) ? p.mu[so] : 0.f;
-    const float s4 = qvalid ? p.s4[so] : 0.f;
-    const float s7d = qvalid ? p.s7d[so] : 0.f;
+    // s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O): each half-lane holds half of the row's
+    // columns of G and dO as B operands; O and TO are read in the same pattern.
+    float s4 = 0.f, s7d = 0.f;
+    {
+        const elem_t* op = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
+        const elem_t* top = HAS_G ? p.to.head(b, h) + (int64_t)qrow * p.to.sl : nullptr;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            const u32x4 ov = load8(op, 16 * c + 8 * hf, p.D, qvalid, vec);
+            u32x4 tov;
+            if constexpr (HAS_G) tov = load8(top, 16 * c + 8 * hf, p.D, qvalid, vec);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float o0 = T::to_float((elem_t)(ov[i] & 0xffffu));
+                const float o1 = T::to_float((elem_t)(ov[i] >> 16));
+                if constexpr (HAS_G) {
+                    const float g0 = T::to_float((elem_t)(gB[c][i] & 0xffffu));
+                    const float g1 = T::to_float((elem_t)(gB[c][i] >> 16));
+                    const float t0 = T::to_float((elem_t)(tov[i] & 0xffffu));
+                    const float t1 = T::to_float((elem_t)(tov[i] >> 16));
+                    s4 += g0 * o0 + g1 * o1;
+                    s7d += g0 * t0 + g1 * t1;
+                }
+                if constexpr (HAS_DO) {
+                    const float d0 = T::to_float((elem_t)(doB[c][i] & 0xffffu));
+                    const float d1 = T::to_float((elem_t)(doB[c][i] >> 16));
+                    s7d += d0 * o0 + d1 * o1;
+                }
+            }
+        }
+        s4 += other_half(s4);
+        s7d += other_half(s7d);
+        if (hf == 0) {  // every row below Lr is written (zeros beyond Lq): the column-owned
+                        // kernel, which runs after this one, stages whole 32-row groups
+            p.lse2[so] = lse2;
+            p.s4[so] = s4;
+            p.s7d[so] = s7d;
+        }
+    }
+    if constexpr (DMA) {
+        // Everything loaded so far has been consumed above except the B operands: retire them
+        // before the first LDS-DMA copy so that wait_vmcnt() only has the ring's traffic to count.
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            asm volatile("" : "+v"(qB[c]));
+            if constexpr (HAS_G) {
+                asm volatile("" : "+v"(tqB[c]));
+                asm volatile("" : "+v"(gB[c]));
+            }
+            if constexpr (HAS_DO) asm volatile("" : "+v"(doB[c]));
+        }
+    }
 
+    SJVP_TS(1);
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = HAS_G ? p.tk.head(b, h) : nullptr;
     const elem_t* tvg = HAS_G ? p.tv.head(b, h) : nullptr;
     const float sl2 = p.scale * kLog2e;
+
+    auto issue = [&](int stage) {
+        elem_t* slot = ring + (stage % R) * SM::slot;
+        const int row0 = stage * kStageRows;
+        fill_slab<HD, DMA>(slot, kg, p.k.sl, row0, p.Lk, p.D, vec, tid);
+        fill_slab<HD, DMA>(slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec, tid);
+        if constexpr (HAS_G) {
+            fill_slab<HD, DMA>(slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec, tid);
+            fill_slab<HD, DMA>(slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec, tid);
+        }
+    };
 
     f32x16 dq[DT], dtq[DT];
 #pragma unroll
@@ -359,73 +178,90 @@ __global__ __launch_bounds__(kThreads) void bwd_row_kernel(const BwdParams p) {
         if constexpr (HAS_G) dtq[t] = f32x16{0};
     }
 
-    for (int k0 = 0; k0 < p.Lk; k0 += BN) {
-        __syncthreads();
-        stage_rows<HD, BN>(sK, kg, p.k.sl, k0, p.Lk, p.D, vec, tid);
-        stage_rows<HD, BN>(sV, vg, p.v.sl, k0, p.Lk, p.D, vec, tid);
-        if constexpr (HAS_G) {
-            stage_rows<HD, BN>(sTK, tkg, p.tk.sl, k0, p.Lk, p.D, vec, tid);
-            stage_rows<HD, BN>(sTV, tvg, p.tv.sl, k0, p.Lk, p.D, vec, tid);
+    auto compute = [&](const elem_t* slot, int k0, auto ragged_tag) {
+        constexpr bool RAGGED = decltype(ragged_tag)::value;
+        const elem_t* sK = slot;
+        const elem_t* sV = slot + Slab<HD>::elems;
+        const elem_t* sTK = slot + 2 * Slab<HD>::elems;
+        const elem_t* sTV = slot + 3 * Slab<HD>::elems;
+        f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            u32x4 ak = lds_a_rows<HD>(sK, c, x, hf);
+            u32x4 av = lds_a_rows<HD>(sV, c, x, hf);
+            s = T::mfma(ak, qB[c], s);
+            if constexpr (HAS_G) {
+                ts = T::mfma(ak, tqB[c], ts);
+                u32x4 atk = lds_a_rows<HD>(sTK, c, x, hf);
+                ts = T::mfma(atk, qB[c], ts);
+                w = T::mfma(av, gB[c], w);
+                u32x4 atv = lds_a_rows<HD>(sTV, c, x, hf);
+                xy = T::mfma(atv, gB[c], xy);
+            }
+            if constexpr (HAS_DO) xy = T::mfma(av, doB[c], xy);
         }
-        __syncthreads();
-        if (!wave_active) continue;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            float pj = fast_exp2(fmaf(s[j], sl2, -lse2));
+            if constexpr (RAGGED) {
+                // keys beyond Lk are zero rows; exp(-lse) may overflow when every real score is
+                // very negative, so their P is forced to zero
+                if (k0 + 8 * (j >> 2) + 4 * hf + (j & 3) >= p.Lk) pj = 0.f;
+            }
+            if constexpr (HAS_G) {
+                const float n = fmaf(ts[j], p.scale, -mu);
+                const float dts = pj * (w[j] - s4);
+                w[j] = dts;
+                xy[j] = fmaf(dts, n, pj * (xy[j] - s7d));
+            } else {
+                xy[j] = pj * (xy[j] - s7d);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const u32x4 dsB = pack_b<T>(xy, c);
+            u32x4 dtsB;
+            if constexpr (HAS_G) dtsB = pack_b<T>(w, c);
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                const u32x4 ak = lds_a_transposed<HD>(sK, c, 32 * d, lane);
+                dq[d] = T::mfma(ak, dsB, dq[d]);
+                if constexpr (HAS_G) {
+                    dtq[d] = T::mfma(ak, dtsB, dtq[d]);
+                    const u32x4 atk = lds_a_transposed<HD>(sTK, c, 32 * d, lane);
+                    dq[d] = T::mfma(atk, dtsB, dq[d]);
+                }
+            }
+        }
+    };
 
-#pragma unroll
-        for (int t = 0; t < BN / 32; ++t) {
-            const int y0 = 32 * t;
-            if (k0 + y0 >= p.Lk) break;
-            // Keys beyond Lk are staged as zero rows of K, K_dot, V, V_dot and their P is forced
-            // to zero below.
-            f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                u32x4 ak = lds_a_rows<HD>(sK, y0, c, x, hf);
-                u32x4 av = lds_a_rows<HD>(sV, y0, c, x, hf);
-                s = T::mfma(ak, qB[c], s);
-                if constexpr (HAS_G) {
-                    ts = T::mfma(ak, tqB[c], ts);
-                    u32x4 atk = lds_a_rows<HD>(sTK, y0, c, x, hf);
-                    ts = T::mfma(atk, qB[c], ts);
-                    w = T::mfma(av, gB[c], w);
-                    u32x4 atv = lds_a_rows<HD>(sTV, y0, c, x, hf);
-                    xy = T::mfma(atv, gB[c], xy);
-                }
-                if constexpr (HAS_DO) xy = T::mfma(av, doB[c], xy);
-            }
-            const bool ragged = (k0 + y0 + 32 > p.Lk);
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                float pj = fast_exp2(s[j] * sl2 - lse2);
-                // exp(-lse) of a padded key may overflow when every real score is very negative
-                if (ragged && k0 + y0 + 8 * (j >> 2) + 4 * hf + (j & 3) >= p.Lk) pj = 0.f;
-                if constexpr (HAS_G) {
-                    const float n = ts[j] * p.scale - mu;
-                    const float dts = pj * (w[j] - s4);
-                    w[j] = dts;
-                    xy[j] = dts * n + pj * (xy[j] - s7d);
-                } else {
-                    xy[j] = pj * (xy[j] - s7d);
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const u32x4 dsB = pack_b<T>(xy, c);
-                u32x4 dtsB;
-                if constexpr (HAS_G) dtsB = pack_b<T>(w, c);
-#pragma unroll
-                for (int d = 0; d < DT; ++d) {
-                    const u32x4 ak = lds_a_transposed<HD>(sK, y0, c, 32 * d, lane);
-                    dq[d] = T::mfma(ak, dsB, dq[d]);
-                    if constexpr (HAS_G) {
-                        dtq[d] = T::mfma(ak, dtsB, dtq[d]);
-                        const u32x4 atk = lds_a_transposed<HD>(sTK, y0, c, 32 * d, lane);
-                        dq[d] = T::mfma(atk, dtsB, dq[d]);
-                    }
-                }
-            }
+    const int n = (p.Lk + kStageRows - 1) / kStageRows;
+    if constexpr (DMA) {
+        for (int s = 0; s < R && s < n; ++s) issue(s);
+    }
+    SJVP_TS(2);
+    for (int i = 0; i < n; ++i) {
+        if constexpr (DMA) {
+            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
+            __syncthreads();
+            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
+            if (i == 0) { SJVP_TS(3); }
+        } else {
+            __syncthreads();
+            issue(i);
+            __syncthreads();
+        }
+        if (!wave_active) continue;
+        const elem_t* slot = ring + (i % R) * SM::slot;
+        const int k0 = i * kStageRows;
+        if (k0 + kStageRows > p.Lk) {
+            compute(slot, k0, std::true_type{});
+        } else {
+            compute(slot, k0, std::false_type{});
         }
     }
 
+    SJVP_TS(4);
     if (!qvalid) return;
     elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
 #pragma unroll
@@ -435,6 +271,262 @@ __global__ __launch_bounds__(kThreads) void bwd_row_kernel(const BwdParams p) {
 #pragma unroll
         for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
     }
+    SJVP_TS_DUMP(p.dbg, 1);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Column-owned kernel: a wavefront owns 32 keys and streams the queries.  DO_K selects dK (and
+// dK_dot), DO_V selects dV (and dV_dot); DT0/NDT select the 32-wide head-dimension tiles that are
+// accumulated (at HD = 128 the work is split to stay inside the register file).
+template <int HD, int R, bool HAS_DO, bool HAS_G>
+struct ColSmem {
+    static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
+    static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
+    static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
+    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
+};
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT,
+          bool DMA>
+__global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd_col_kernel(
+    const BwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    using SM = ColSmem<HD, R, HAS_DO, HAS_G>;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    // slot layout: Q | [Q_dot | G] | [dO] | stats(lse2, mu, s4, s7d)
+    constexpr int oTQ = Slab<HD>::elems;
+    constexpr int oG = 2 * Slab<HD>::elems;
+    constexpr int oDO = (HAS_G ? 3 : 1) * Slab<HD>::elems;
+    constexpr int oST = SM::nt * Slab<HD>::elems;
+
+    constexpr int KC = HD / 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int x = lane & 31;
+    const int hf = lane >> 5;
+    const int bh = blockIdx.x / p.k_blocks;
+    const int kb = blockIdx.x % p.k_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const bool vec = p.vec != 0;
+    // LDS-DMA instructions per stage issued by this wave: the tensors, plus one 4-byte copy of two
+    // statistic arrays by waves 0 and 1
+    const int spt = SM::nt * Slab<HD>::per_thread + (wave < 2 ? 1 : 0);
+
+    SJVP_TS_DECL;
+    SJVP_TS(0);
+    const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
+    const bool kvalid = krow < p.Lk;
+    const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;
+
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    {
+        const elem_t* kp = p.k.head(b, h) + (int64_t)krow * p.k.sl;
+        const elem_t* vp = p.v.head(b, h) + (int64_t)krow * p.v.sl;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            kB[c] = load8(kp, 16 * c + 8 * hf, p.D, kvalid, vec);
+            if constexpr (DO_K) vB[c] = load8(vp, 16 * c + 8 * hf, p.D, kvalid, vec);
+        }
+        if constexpr (HAS_G) {
+            const elem_t* tkp = p.tk.head(b, h) + (int64_t)krow * p.tk.sl;
+            const elem_t* tvp = p.tv.head(b, h) + (int64_t)krow * p.tv.sl;
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                tkB[c] = load8(tkp, 16 * c + 8 * hf, p.D, kvalid, vec);
+                if constexpr (DO_K) tvB[c] = load8(tvp, 16 * c + 8 * hf, p.D, kvalid, vec);
+            }
+        }
+        if constexpr (DMA) {
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                asm volatile("" : "+v"(kB[c]));
+                if constexpr (DO_K) asm volatile("" : "+v"(vB[c]));
+                if constexpr (HAS_G) {
+                    asm volatile("" : "+v"(tkB[c]));
+                    if constexpr (DO_K) asm volatile("" : "+v"(tvB[c]));
+                }
+            }
+        }
+    }
+
+    SJVP_TS(1);
+    const elem_t* qg = p.q.head(b, h);
+    const elem_t* tqg = HAS_G ? p.tq.head(b, h) : nullptr;
+    const elem_t* gg = HAS_G ? p.dTO.head(b, h) : nullptr;
+    const elem_t* dog = HAS_DO ? p.dO.head(b, h) : nullptr;
+    const float sl2 = p.scale * kLog2e;
+
+    auto issue = [&](int stage) {
+        elem_t* slot = ring + (stage % R) * SM::slot;
+        const int row0 = stage * kStageRows;
+        fill_slab<HD, DMA>(slot, qg, p.q.sl, row0, p.Lq, p.D, vec, tid);
+        if constexpr (HAS_G) {
+            fill_slab<HD, DMA>(slot + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec, tid);
+            fill_slab<HD, DMA>(slot + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec, tid);
+        }
+        if constexpr (HAS_DO) fill_slab<HD, DMA>(slot + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec, tid);
+        // Row statistics of the stage (rows < Lr are defined in all four arrays; rows beyond Lq
+        // hold finite values and multiply zero rows of Q, Q_dot, G, dO below).
+        float* st = reinterpret_cast<float*>(slot + oST);
+        const int64_t so = (int64_t)bh * p.Lr + row0 + (lane & 31);
+        if (wave < 2) {
+            const float* src = wave == 0 ? (hf == 0 ? p.lse2 : p.mu) : (hf == 0 ? p.s4 : p.s7d);
+            if constexpr (DMA) {
+                const uint32_t base = lds_addr(st) + (uint32_t)(wave * 64 * 4);
+                if (HAS_G || !(wave == 0 && hf == 1)) dma4(src + so, base);
+            } else {
+                st[wave * 64 + lane] = (HAS_G || !(wave == 0 && hf == 1)) ? src[so] : 0.f;
+            }
+        }
+    };
+
+    f32x16 dk[NDT], dv[NDT], dtk[NDT], dtv[NDT];
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) {
+        if constexpr (DO_K) dk[t] = f32x16{0};
+        if constexpr (DO_V) dv[t] = f32x16{0};
+        if constexpr (HAS_G) {
+            if constexpr (DO_K) dtk[t] = f32x16{0};
+            if constexpr (DO_V) dtv[t] = f32x16{0};
+        }
+    }
+
+    auto compute = [&](const elem_t* slot) {
+        const elem_t* sQ = slot;
+        const elem_t* sTQ = slot + oTQ;
+        const elem_t* sG = slot + oG;
+        const elem_t* sDO = slot + oDO;
+        const float* sStat = reinterpret_cast<const float*>(slot + oST);
+        // tiles: rows = queries (registers), columns = this wave's keys (lanes)
+        f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            u32x4 aq = lds_a_rows<HD>(sQ, c, x, hf);
+            s = T::mfma(aq, kB[c], s);
+            if constexpr (HAS_G) {
+                ts = T::mfma(aq, tkB[c], ts);
+                u32x4 atq = lds_a_rows<HD>(sTQ, c, x, hf);
+                ts = T::mfma(atq, kB[c], ts);
+                if constexpr (DO_K) {
+                    u32x4 ag = lds_a_rows<HD>(sG, c, x, hf);
+                    w = T::mfma(ag, vB[c], w);
+                    xy = T::mfma(ag, tvB[c], xy);
+                }
+            }
+            if constexpr (HAS_DO && DO_K) {
+                u32x4 ado = lds_a_rows<HD>(sDO, c, x, hf);
+                xy = T::mfma(ado, vB[c], xy);
+            }
+        }
+        // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int r0 = 8 * jj + 4 * hf;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+            const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+            const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+            const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = 4 * jj + i;
+                const float pj = fast_exp2(fmaf(s[j], sl2, -lse4[i]));
+                s[j] = pj;
+                if constexpr (HAS_G) {
+                    const float n = fmaf(ts[j], p.scale, -mu4[i]);
+                    if constexpr (DO_K) {
+                        const float dts = pj * (w[j] - s44[i]);
+                        w[j] = dts;
+                        xy[j] = fmaf(dts, n, pj * (xy[j] - s74[i]));
+                    }
+                    if constexpr (DO_V) ts[j] = pj * n;
+                } else if constexpr (DO_K) {
+                    xy[j] = pj * (xy[j] - s74[i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            u32x4 pB, dsB, pdB, dtsB;
+            if constexpr (DO_V) pB = pack_b<T>(s, c);
+            if constexpr (DO_K) dsB = pack_b<T>(xy, c);
+            if constexpr (HAS_G) {
+                if constexpr (DO_V) pdB = pack_b<T>(ts, c);
+                if constexpr (DO_K) dtsB = pack_b<T>(w, c);
+            }
+#pragma unroll
+            for (int d = 0; d < NDT; ++d) {
+                const int d0 = 32 * (DT0 + d);
+                if constexpr (DO_K) {
+                    const u32x4 aq = lds_a_transposed<HD>(sQ, c, d0, lane);
+                    dk[d] = T::mfma(aq, dsB, dk[d]);
+                    if constexpr (HAS_G) {
+                        dtk[d] = T::mfma(aq, dtsB, dtk[d]);
+                        const u32x4 atq = lds_a_transposed<HD>(sTQ, c, d0, lane);
+                        dk[d] = T::mfma(atq, dtsB, dk[d]);
+                    }
+                }
+                if constexpr (DO_V) {
+                    if constexpr (HAS_G) {
+                        const u32x4 ag = lds_a_transposed<HD>(sG, c, d0, lane);
+                        dtv[d] = T::mfma(ag, pB, dtv[d]);
+                        dv[d] = T::mfma(ag, pdB, dv[d]);
+                    }
+                    if constexpr (HAS_DO) {
+                        const u32x4 ado = lds_a_transposed<HD>(sDO, c, d0, lane);
+                        dv[d] = T::mfma(ado, pB, dv[d]);
+                    }
+                }
+            }
+        }
+    };
+
+    const int n = (p.Lq + kStageRows - 1) / kStageRows;
+    if constexpr (DMA) {
+        for (int s = 0; s < R && s < n; ++s) issue(s);
+    }
+    SJVP_TS(2);
+    for (int i = 0; i < n; ++i) {
+        if constexpr (DMA) {
+            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * spt);
+            __syncthreads();
+            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
+            if (i == 0) { SJVP_TS(3); }
+        } else {
+            __syncthreads();
+            issue(i);
+            __syncthreads();
+        }
+        if (!wave_active) continue;
+        compute(ring + (i % R) * SM::slot);
+    }
+
+    SJVP_TS(4);
+    if (!kvalid) return;
+    if constexpr (DO_K) {
+        elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;
+#pragma unroll
+        for (int d = 0; d < NDT; ++d)
+            store_acc<T>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
+        if constexpr (HAS_G) {
+            elem_t* dtkrow = p.dtk.head(b, h) + (int64_t)krow * p.dtk.sl;
+#pragma unroll
+            for (int d = 0; d < NDT; ++d)
+                store_acc<T>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
+        }
+    }
+    if constexpr (DO_V) {
+        elem_t* dvrow = p.dv.head(b, h) + (int64_t)krow * p.dv.sl;
+#pragma unroll
+        for (int d = 0; d < NDT; ++d) store_acc<T>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
+        if constexpr (HAS_G) {
+            elem_t* dtvrow = p.dtv.head(b, h) + (int64_t)krow * p.dtv.sl;
+#pragma unroll
+            for (int d = 0; d < NDT; ++d)
+                store_acc<T>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
+        }
+    }
+    SJVP_TS_DUMP(p.dbg, 2);
 }
 
 }  // namespace sjvp

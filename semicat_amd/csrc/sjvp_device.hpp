@@ -4,7 +4,7 @@
 // --------------------------------------------
 // One wavefront (64 lanes) owns 32 positions of one sequence axis ("owned" axis X: queries in the
 // forward and in the dQ kernel, keys in the dK/dV kernel) and walks over the other axis ("looped"
-// axis Y) in tiles of 32.  Every score-like 32x32 tile is produced by
+// axis Y) in stages of 32 rows.  Every score-like 32x32 tile is produced by
 //     v_mfma_f32_32x32x16_{bf16,f16}:  C[y][x] += sum_d A[y][d] * B[d][x]
 // with A read row-major from LDS (the looped side) and B held in registers (the owned side), so
 // that in the accumulator lane l holds column x = l % 32 and, in register j, row
@@ -12,11 +12,40 @@
 // Per-x quantities (softmax max/sum, row statistics) are then per-lane scalars, and the tile,
 // converted to 16-bit in place, is already the B operand (k = y) of the next contraction
 //     OUT^T[d][x] += sum_y A'[d][y] * Tile[y][x],
-// whose A' = (looped-side tensor)^T is fetched from the same row-major LDS tile with the
+// whose A' = (looped-side tensor)^T is fetched from the same row-major LDS stage with the
 // transposing LDS read ds_read_b64_tr_b16.  No tile ever goes through LDS or shuffles.
+//
+// Streaming
+// ---------
+// The looped side is streamed through a ring of LDS slots.  On the fast path the copy is done by
+// the LDS-DMA form of the global load (global_load_lds_dwordx4: 16 bytes per lane straight into
+// LDS, no registers), issued several stages ahead and retired with explicit s_waitcnt vmcnt(n), so
+// that HBM traffic overlaps the MFMA work of earlier stages.  A stage slab is unpadded ([32][HD]
+// 16-bit) and XOR-swizzled in units of 16 bytes, which keeps both LDS access patterns (row-major
+// 16-byte reads of 8 consecutive rows, and the 4-row x 32-byte footprint of a transposing read)
+// free of bank conflicts; because every lane of an LDS-DMA load supplies its own global address,
+// the swizzle costs nothing at copy time.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#ifdef SJVP_X_TIMING
+#define SJVP_TS_DECL unsigned long long tstamp[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define SJVP_TS(i) tstamp[i] = __builtin_readcyclecounter()
+#define SJVP_TS_DUMP(dbg, kid)                                                              \
+    do {                                                                                    \
+        __builtin_amdgcn_s_waitcnt(0);                                                      \
+        SJVP_TS(5);                                                                         \
+        if ((threadIdx.x & 63) == 0 && (dbg)) {                                             \
+            unsigned long long* d_ = (dbg) + ((size_t)(kid) * 4096 + blockIdx.x * 4 + (threadIdx.x >> 6)) * 8; \
+            for (int i_ = 0; i_ < 6; ++i_) d_[i_] = tstamp[i_];                             \
+        }                                                                                   \
+    } while (0)
+#else
+#define SJVP_TS_DECL
+#define SJVP_TS(i)
+#define SJVP_TS_DUMP(dbg, kid)
+#endif
 
 namespace sjvp {
 
@@ -34,6 +63,7 @@ typedef uint16_t elem_t;  // storage type of one 16-bit element, whatever its fo
 constexpr int kThreads = 256;  // 4 wavefronts per workgroup
 constexpr int kWaves = 4;
 constexpr int kOwned = 32 * kWaves;  // positions of the owned axis per workgroup
+constexpr int kStageRows = 32;       // rows of the looped axis per stage
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -74,6 +104,12 @@ struct TensorView {
     }
 };
 
+struct OutView {
+    elem_t* ptr;
+    int64_t sb, sh, sl;
+    __device__ __forceinline__ elem_t* head(int b, int h) const { return ptr + b * sb + h * sh; }
+};
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -109,51 +145,116 @@ __device__ __forceinline__ void store4(elem_t* row, int d, int D, u32x2 val, boo
     }
 }
 
-// LDS row pitch (elements) of a staged [rows][HD] tile.  The 16-element pad makes the pitch
-// 8 banks (mod 32) so that the four rows touched by one 16-lane group of a transposing read fall
-// into disjoint banks.
+// ---------------------------------------------------------------------------------------------
+// LDS stage slab: [32 rows][HD] elements, 16-byte chunk c of row r stored at chunk position
+// c ^ swz(r).  Over 8 consecutive rows swz is a permutation of 0..7 (row-major 16-byte reads of a
+// fixed logical chunk hit 8 distinct positions), and over 4 consecutive rows starting at a multiple
+// of 4 the positions of a fixed chunk pair fall into 4 distinct 32-byte regions (transposing read).
 template <int HD>
-struct Pitch {
-    static constexpr int value = HD + 16;
+__device__ __forceinline__ int swz(int row) {
+    if constexpr (HD == 32) return (((row >> 1) & 1) << 1) | ((row >> 2) & 1);
+    return ((row & 3) << 1) | ((row >> 2) & 1);
+}
+
+template <int HD>
+struct Slab {
+    static constexpr int elems = kStageRows * HD;
+    static constexpr int chunks = kStageRows * HD / 8;  // 16-byte chunks
+    static constexpr int per_thread = (chunks + kThreads - 1) / kThreads;
 };
 
-// Cooperative global -> LDS copy of ROWS rows (row0 .. row0+ROWS-1 of a [L][D] head slice) into a
-// row-major LDS tile, zero-filled beyond L and beyond D.
-template <int HD, int ROWS>
-__device__ __forceinline__ void stage_rows(elem_t* lds, const elem_t* g, int64_t sl, int row0,
-                                           int L, int D, bool vec, int tid) {
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+// LDS-DMA: each active lane copies 16 bytes from its global address to LDS byte address
+// base + 16 * lane_id (base must be wave-uniform).  Completion is tracked by vmcnt only.
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+// 4-byte form: LDS byte address base + 4 * lane_id.
+__device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
+                 :
+                 : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
+                 : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) for a run-time n (clamped to the encodable 0..63): at most n of this wave's
+// vector-memory operations may still be outstanding afterwards.  Loads and LDS-DMA copies retire
+// in issue order, so this guarantees that all but the n most recent ones have landed.
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define SJVP_VM(k) \
+    case k: __builtin_amdgcn_s_waitcnt(((k) & 15) | (((k) >> 4) << 14) | 0x0F70); break;
+    switch (n) {
+        SJVP_VM(0) SJVP_VM(1) SJVP_VM(2) SJVP_VM(3) SJVP_VM(4) SJVP_VM(5) SJVP_VM(6) SJVP_VM(7)
+        SJVP_VM(8) SJVP_VM(9) SJVP_VM(10) SJVP_VM(11) SJVP_VM(12) SJVP_VM(13) SJVP_VM(14)
+        SJVP_VM(15) SJVP_VM(16) SJVP_VM(17) SJVP_VM(18) SJVP_VM(19) SJVP_VM(20) SJVP_VM(21)
+        SJVP_VM(22) SJVP_VM(23) SJVP_VM(24) SJVP_VM(25) SJVP_VM(26) SJVP_VM(27) SJVP_VM(28)
+        SJVP_VM(29) SJVP_VM(30) SJVP_VM(31) SJVP_VM(32) SJVP_VM(33) SJVP_VM(34) SJVP_VM(35)
+        SJVP_VM(36) SJVP_VM(37) SJVP_VM(38) SJVP_VM(39) SJVP_VM(40) SJVP_VM(41) SJVP_VM(42)
+        SJVP_VM(43) SJVP_VM(44) SJVP_VM(45) SJVP_VM(46) SJVP_VM(47) SJVP_VM(48)
+        default: __builtin_amdgcn_s_waitcnt(0x0F70 | 15 | (3 << 14)); break;  // vmcnt(63)
+    }
+#undef SJVP_VM
+}
+
+// Copy stage rows row0 .. row0+31 of one [L][D] head slice into a slab (swizzled), zero-filled
+// beyond L and beyond D.  DMA = true: asynchronous LDS-DMA (needs `vec` inputs); the caller retires
+// it with wait_vmcnt + barrier; exactly Slab<HD>::per_thread LDS-DMA instructions are issued by
+// every wave when HD >= 64.  DMA = false: synchronous copy through registers (any alignment).
+template <int HD, bool DMA>
+__device__ __forceinline__ void fill_slab(elem_t* slab, const elem_t* g, int64_t sl, int row0, int L,
+                                          int D, bool vec, int tid) {
     constexpr int CH = HD / 8;
-    constexpr int P = Pitch<HD>::value;
 #pragma unroll
-    for (int id = tid; id < ROWS * CH; id += kThreads) {
-        int r = id / CH, c = id % CH;
-        int row = row0 + r;
-        u32x4 val = load8(g + (int64_t)row * sl, c * 8, D, row < L, vec);
-        *reinterpret_cast<u32x4*>(lds + r * P + c * 8) = val;
+    for (int i = 0; i < Slab<HD>::per_thread; ++i) {
+        const int pos = tid + i * kThreads;  // chunk position inside the slab
+        if (Slab<HD>::chunks % kThreads != 0 && pos >= Slab<HD>::chunks) break;
+        const int r = pos / CH;
+        const int c = (pos % CH) ^ swz<HD>(r);
+        const int row = row0 + r;
+        const bool valid = (row < L) && (8 * c < D);
+        if constexpr (DMA) {
+            // every lane of the wave writes base + 16*lane: base is the slab address of the wave's
+            // first chunk position
+            const uint32_t base = lds_addr(slab) + (uint32_t)((pos & ~63) * 16);
+            if (valid) {
+                dma16(g + (int64_t)row * sl + 8 * c, base);
+            } else {
+                *reinterpret_cast<u32x4*>(slab + pos * 8) = u32x4{0u, 0u, 0u, 0u};
+            }
+        } else {
+            *reinterpret_cast<u32x4*>(slab + pos * 8) = load8(g + (int64_t)row * sl, 8 * c, D, row < L, vec);
+        }
     }
 }
 
-// A operand (32 rows y0..y0+31 of the looped side, k = d chunk c) read row-major from LDS.
+// A operand (the 32 rows of a slab, k = d chunk cc of 16) read row-major.
 template <int HD>
-__device__ __forceinline__ u32x4 lds_a_rows(const elem_t* lds, int y0, int c, int x, int hf) {
-    return *reinterpret_cast<const u32x4*>(lds + (y0 + x) * Pitch<HD>::value + 16 * c + 8 * hf);
+__device__ __forceinline__ u32x4 lds_a_rows(const elem_t* slab, int cc, int x, int hf) {
+    return *reinterpret_cast<const u32x4*>(slab + x * HD + (((2 * cc + hf) ^ swz<HD>(x)) << 3));
 }
 
-// A operand of the transposed use: A'[d][y] for d = d0 + x and the eight looped positions that the
-// lane's half owns in k-chunk c of a score tile, i.e. y0 + 16c + 4hf + {0..3} and + 8 more.  Read
-// with two ds_read_b64_tr_b16: within each group of 16 lanes, lane 4j+g supplies the address of row
+// A operand of the transposed use: A'[d][y] for d = d0 + x and the eight slab rows that the lane's
+// half owns in k-chunk c of a score tile, i.e. 16c + 4hf + {0..3} and + 8 more.  Read with two
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane 4j+g supplies the address of row
 // (k0 + j), columns 4g..4g+3, and lane i receives column i of those four rows.
 template <int HD>
-__device__ __forceinline__ u32x4 lds_a_transposed(const elem_t* lds, int y0, int c, int d0, int lane) {
-    constexpr int P = Pitch<HD>::value;
+__device__ __forceinline__ u32x4 lds_a_transposed(const elem_t* slab, int c, int d0, int lane) {
     const int hf = lane >> 5;
     const int i16 = lane & 15;
-    const int xb = lane & 16;  // 0 or 16: which half of the 32 output rows d this 16-lane group feeds
-    const int krow = y0 + 16 * c + 4 * hf + (i16 >> 2);
-    const elem_t* p0 = lds + krow * P + d0 + xb + 4 * (i16 & 3);
+    const int xb = lane & 16;  // which half of the 32 output rows d this 16-lane group feeds
+    const int krow = 16 * c + 4 * hf + (i16 >> 2);
+    const int e = d0 + xb + 4 * (i16 & 3);  // logical element (column) offset, multiple of 4
+    const elem_t* p0 = slab + krow * HD + (((e >> 3) ^ swz<HD>(krow)) << 3) + (e & 7);
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    // rows krow and krow + 8 share their swizzle (it depends on row mod 8 only)
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 8 * P));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 8 * HD));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo);
     u32x2 h2 = __builtin_bit_cast(u32x2, hi);
     u32x4 r = {l2[0], l2[1], h2[0], h2[1]};
@@ -180,6 +281,13 @@ __device__ __forceinline__ void store_acc(elem_t* row, int d0, int hf, int D, co
                      T::pack2(acc[4 * jj + 2] * mul, acc[4 * jj + 3] * mul)};
         store4(row, d0 + 8 * jj + 4 * hf, D, val, vec);
     }
+}
+
+// Ring schedule shared by the streaming kernels: stages 0..n-1, R slots, stage s lives in slot
+// s % R.  Before consuming stage i the kernel has issued stages 0 .. issued_before(i)-1.
+__device__ __forceinline__ int ring_issued_before(int i, int R, int n) {
+    const int upto = (i == 0) ? R : i - 1 + R;
+    return upto < n ? upto : n;
 }
 
 }  // namespace sjvp

@@ -3,20 +3,20 @@
 // Computes what semicat/jvp_utils/ryu_triton.py:73-291 computes - O, TO, M (= lse), MU, LI in one
 // online-softmax pass - with a different decomposition: a workgroup of four wavefronts owns 128
 // query rows of one (batch, head); each wavefront owns 32 of them as MFMA columns and walks over
-// the keys in tiles of 32 staged in LDS (K, K_dot, V, V_dot row-major, shared by the four waves).
-// Scores are produced transposed (S^T = K Q^T) so that the running maximum, the exp-sum and mu are
-// per-lane scalars and the probability tile is directly the B operand of O^T += V^T P^T.
+// the keys in stages of 32 streamed through an LDS ring (K, V, K_dot, V_dot; shared by the four
+// waves).  Scores are produced transposed (S^T = K Q^T) so that the running maximum, the exp-sum
+// and mu are per-lane scalars and the probability tile is directly the B operand of
+// O^T += V^T P^T.
 #pragma once
+#include <type_traits>
+
 #include "sjvp_device.hpp"
 
 namespace sjvp {
 
 struct FwdParams {
     TensorView q, k, v, tq, tk, tv;
-    elem_t* o;
-    int64_t o_sb, o_sh, o_sl;
-    elem_t* to;
-    int64_t to_sb, to_sh, to_sl;
+    OutView o, to;
     float* lse;
     float* mu;
     float* li;
@@ -24,28 +24,37 @@ struct FwdParams {
     int q_blocks;  // ceil(Lq / 128)
     float scale;
     int vec;  // all tensors 16-byte aligned, strides % 8 == 0, D % 8 == 0
+#ifdef SJVP_X_TIMING
+    unsigned long long* dbg;
+#endif
 };
 
-template <int HD, int BN, bool JVP>
+template <int HD, int R, bool JVP>
 struct FwdSmem {
-    static constexpr int tile = BN * Pitch<HD>::value;          // elements per staged tensor
-    static constexpr int bytes = (JVP ? 4 : 2) * tile * (int)sizeof(elem_t);
+    static constexpr int nt = JVP ? 4 : 2;                      // tensors per stage
+    static constexpr int slot = nt * Slab<HD>::elems;            // elements per ring slot
+    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, int BN, bool JVP>
-__global__ __launch_bounds__(kThreads) void fwd_kernel(const FwdParams p) {
+// The reference maximum of the online softmax is only raised when a new tile exceeds it by more
+// than this many log2 units.  Any reference point is valid as long as exp2 stays in range: the
+// unnormalised probabilities are then bounded by 2^kMaxSlack instead of 1 and the final division
+// by the exp-sum is unaffected.  This keeps the accumulator rescale out of almost every tile.
+constexpr float kMaxSlack = 6.0f;
+
+template <typename T, int HD, int R, bool JVP, bool DMA>
+__global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    elem_t* sK = reinterpret_cast<elem_t*>(smem_raw);
-    elem_t* sV = sK + FwdSmem<HD, BN, JVP>::tile;
-    elem_t* sTK = sV + FwdSmem<HD, BN, JVP>::tile;
-    elem_t* sTV = sTK + FwdSmem<HD, BN, JVP>::tile;
+    using SM = FwdSmem<HD, R, JVP>;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
 
     constexpr int KC = HD / 16;  // k-chunks of the score contraction
     constexpr int DT = HD / 32;  // 32-wide tiles of the head dimension
+    constexpr int SPT = SM::nt * Slab<HD>::per_thread;  // LDS-DMA instructions per thread per stage
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int x = lane & 31;
     const int hf = lane >> 5;
 
@@ -54,6 +63,8 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(const FwdParams p) {
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
 
+    SJVP_TS_DECL;
+    SJVP_TS(0);
     const int qrow = qb * kOwned + wave * 32 + x;  // the query this lane owns
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -69,114 +80,149 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int c = 0; c < KC; ++c) tqB[c] = load8(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
+        if constexpr (DMA) {
+            // Retire these loads before the first LDS-DMA copy is issued: afterwards the only
+            // vector-memory traffic in flight is the ring's, which wait_vmcnt() counts.
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                asm volatile("" : "+v"(qB[c]));
+                if constexpr (JVP) asm volatile("" : "+v"(tqB[c]));
+            }
+        }
     }
 
+    SJVP_TS(1);
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = JVP ? p.tk.head(b, h) : nullptr;
     const elem_t* tvg = JVP ? p.tv.head(b, h) : nullptr;
 
-    // log2-domain softmax: s2 = S * scale * log2(e)
+    auto issue = [&](int stage) {
+        elem_t* slot = ring + (stage % R) * SM::slot;
+        const int row0 = stage * kStageRows;
+        fill_slab<HD, DMA>(slot, kg, p.k.sl, row0, p.Lk, p.D, vec, tid);
+        fill_slab<HD, DMA>(slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec, tid);
+        if constexpr (JVP) {
+            fill_slab<HD, DMA>(slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec, tid);
+            fill_slab<HD, DMA>(slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec, tid);
+        }
+    };
+
+    // log2-domain softmax: exponent = S * (scale*log2 e) - m
     const float sl2 = p.scale * kLog2e;
-    float m_i = -INFINITY;  // running max (same in both half-lanes of a query)
-    float l_i = 0.f;        // exp-sum over the keys this half-lane has seen
-    float mu_i = 0.f;       // sum of p * S_dot over the same keys
-    f32x16 acc[DT], gacc[DT], pacc[DT];
+    float m_i = -INFINITY;    // reference maximum (same in both half-lanes of a query)
+    float m_true = -INFINITY; // true running maximum (only needed to report LI)
+    float l_i = 0.f;          // exp-sum over the keys this half-lane has seen
+    float mu_i = 0.f;         // sum of p * S_dot over the same keys
+    // acc = sum P~ V;  tacc = sum (P~ * S_dot) V + P~ V_dot  (the reference's g_acc + p_tv_acc, which
+    // only ever appear added together, ryu_triton.py:274-275)
+    f32x16 acc[DT], tacc[DT];
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
         acc[t] = f32x16{0};
-        if constexpr (JVP) {
-            gacc[t] = f32x16{0};
-            pacc[t] = f32x16{0};
-        }
+        if constexpr (JVP) tacc[t] = f32x16{0};
     }
 
-    for (int k0 = 0; k0 < p.Lk; k0 += BN) {
-        __syncthreads();  // previous stage fully consumed
-        stage_rows<HD, BN>(sK, kg, p.k.sl, k0, p.Lk, p.D, vec, tid);
-        stage_rows<HD, BN>(sV, vg, p.v.sl, k0, p.Lk, p.D, vec, tid);
-        if constexpr (JVP) {
-            stage_rows<HD, BN>(sTK, tkg, p.tk.sl, k0, p.Lk, p.D, vec, tid);
-            stage_rows<HD, BN>(sTV, tvg, p.tv.sl, k0, p.Lk, p.D, vec, tid);
+    auto compute = [&](const elem_t* slot, int k0, auto ragged_tag) {
+        constexpr bool RAGGED = decltype(ragged_tag)::value;
+        const elem_t* sK = slot;
+        const elem_t* sV = slot + Slab<HD>::elems;
+        const elem_t* sTK = slot + 2 * Slab<HD>::elems;
+        const elem_t* sTV = slot + 3 * Slab<HD>::elems;
+        f32x16 s = {0}, ts = {0};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            u32x4 a = lds_a_rows<HD>(sK, c, x, hf);
+            s = T::mfma(a, qB[c], s);
+            if constexpr (JVP) {
+                ts = T::mfma(a, tqB[c], ts);
+                u32x4 at = lds_a_rows<HD>(sTK, c, x, hf);
+                ts = T::mfma(at, qB[c], ts);
+            }
         }
-        __syncthreads();
-        if (!wave_active) continue;
-
+        if constexpr (RAGGED) {
+            // keys beyond Lk are zero rows in LDS (their S_dot is already 0)
 #pragma unroll
-        for (int t = 0; t < BN / 32; ++t) {
-            const int y0 = 32 * t;
-            if (k0 + y0 >= p.Lk) break;
-            f32x16 s = {0}, ts = {0};
+            for (int j = 0; j < 16; ++j)
+                if (k0 + 8 * (j >> 2) + 4 * hf + (j & 3) >= p.Lk) s[j] = -INFINITY;
+        }
+        float mloc = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
 #pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                u32x4 a = lds_a_rows<HD>(sK, y0, c, x, hf);
-                s = T::mfma(a, qB[c], s);
-                if constexpr (JVP) {
-                    ts = T::mfma(a, tqB[c], ts);
-                    u32x4 at = lds_a_rows<HD>(sTK, y0, c, x, hf);
-                    ts = T::mfma(at, qB[c], ts);
-                }
-            }
-            const bool ragged = (k0 + y0 + 32 > p.Lk);
-            float mloc = -INFINITY;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                float sv = s[j] * sl2;
-                if (ragged) {
-                    int key = k0 + y0 + 8 * (j >> 2) + 4 * hf + (j & 3);
-                    if (key >= p.Lk) {
-                        sv = -INFINITY;
-                        if constexpr (JVP) ts[j] = 0.f;
-                    }
-                }
-                s[j] = sv;
-                mloc = fmaxf(mloc, sv);
-            }
-            mloc = fmaxf(mloc, other_half(mloc));
+        for (int j = 4; j < 16; j += 4)
+            mloc = fmaxf(mloc, fmaxf(fmaxf(s[j], s[j + 1]), fmaxf(s[j + 2], s[j + 3])));
+        mloc = fmaxf(mloc, other_half(mloc)) * sl2;
+        m_true = fmaxf(m_true, mloc);
+        if (__builtin_amdgcn_ballot_w64(mloc > m_i + kMaxSlack) != 0) {  // wave-uniform branch
             const float m_new = fmaxf(m_i, mloc);
-            const float alpha = fast_exp2(m_i - m_new);
+            const float alpha = fast_exp2(m_i - m_new);  // 0 on the first tile
             m_i = m_new;
-            float lsum = 0.f, musum = 0.f;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                float pj = fast_exp2(s[j] - m_new);
-                s[j] = pj;
-                lsum += pj;
-                if constexpr (JVP) {
-                    float pt = pj * (ts[j] * p.scale);
-                    ts[j] = pt;
-                    musum += pt;
-                }
-            }
-            l_i = l_i * alpha + lsum;
-            if constexpr (JVP) mu_i = mu_i * alpha + musum;
+            l_i *= alpha;
+            if constexpr (JVP) mu_i *= alpha;
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
                 acc[d] *= alpha;
-                if constexpr (JVP) {
-                    gacc[d] *= alpha;
-                    pacc[d] *= alpha;
-                }
+                if constexpr (JVP) tacc[d] *= alpha;
             }
+        }
+        float lsum = 0.f, musum = 0.f;
 #pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                u32x4 pb = pack_b<T>(s, c);
-                u32x4 ptb;
-                if constexpr (JVP) ptb = pack_b<T>(ts, c);
+        for (int j = 0; j < 16; ++j) {
+            const float pj = fast_exp2(fmaf(s[j], sl2, -m_i));
+            s[j] = pj;
+            lsum += pj;
+            if constexpr (JVP) {
+                const float pt = pj * (ts[j] * p.scale);
+                ts[j] = pt;
+                musum += pt;
+            }
+        }
+        l_i += lsum;
+        if constexpr (JVP) mu_i += musum;
 #pragma unroll
-                for (int d = 0; d < DT; ++d) {
-                    u32x4 av = lds_a_transposed<HD>(sV, y0, c, 32 * d, lane);
-                    acc[d] = T::mfma(av, pb, acc[d]);
-                    if constexpr (JVP) {
-                        gacc[d] = T::mfma(av, ptb, gacc[d]);
-                        u32x4 atv = lds_a_transposed<HD>(sTV, y0, c, 32 * d, lane);
-                        pacc[d] = T::mfma(atv, pb, pacc[d]);
-                    }
+        for (int c = 0; c < 2; ++c) {
+            u32x4 pb = pack_b<T>(s, c);
+            u32x4 ptb;
+            if constexpr (JVP) ptb = pack_b<T>(ts, c);
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                u32x4 av = lds_a_transposed<HD>(sV, c, 32 * d, lane);
+                acc[d] = T::mfma(av, pb, acc[d]);
+                if constexpr (JVP) {
+                    tacc[d] = T::mfma(av, ptb, tacc[d]);
+                    u32x4 atv = lds_a_transposed<HD>(sTV, c, 32 * d, lane);
+                    tacc[d] = T::mfma(atv, pb, tacc[d]);
                 }
             }
         }
+    };
+
+    const int n = (p.Lk + kStageRows - 1) / kStageRows;
+    if constexpr (DMA) {
+        for (int s = 0; s < R && s < n; ++s) issue(s);
+    }
+    SJVP_TS(2);
+    for (int i = 0; i < n; ++i) {
+        if constexpr (DMA) {
+            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
+            __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
+            if (i == 0) { SJVP_TS(3); }
+        } else {
+            __syncthreads();
+            issue(i);
+            __syncthreads();
+        }
+        if (!wave_active) continue;
+        const elem_t* slot = ring + (i % R) * SM::slot;
+        const int k0 = i * kStageRows;
+        if (k0 + kStageRows > p.Lk) {
+            compute(slot, k0, std::true_type{});
+        } else {
+            compute(slot, k0, std::false_type{});
+        }
     }
 
+    SJVP_TS(4);
     if (!wave_active) {
         // All 32 rows of this wave lie beyond Lq: their statistic rows get the values a zero
         // query row produces (and the reference initialises them with): log(Lk), 0, Lk.
@@ -201,25 +247,28 @@ __global__ __launch_bounds__(kThreads) void fwd_kernel(const FwdParams p) {
         const int64_t so = (int64_t)bh * p.Lr + qrow;
         p.lse[so] = (m_i + fast_log2(l)) * kLn2;
         if constexpr (JVP) p.mu[so] = mu_un * inv_l;
-        if (p.li) p.li[so] = l;
+        // LI is the exp-sum relative to the true row maximum (ryu_triton.py:291); l is relative
+        // to m_i, which may lag behind it by up to kMaxSlack.
+        if (p.li) p.li[so] = l * fast_exp2(m_i - m_true);
     }
     if (!qvalid) return;
 
-    elem_t* orow = p.o + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+    elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
 #pragma unroll
     for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
     if constexpr (JVP) {
         // TO = (g_acc - mu_un * O + p_tv_acc) / l     (ryu_triton.py:274-275)
-        elem_t* trow = p.to + b * p.to_sb + h * p.to_sh + (int64_t)qrow * p.to_sl;
+        elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
         const float cmu = mu_un * inv_l;
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
             f32x16 t;
 #pragma unroll
-            for (int j = 0; j < 16; ++j) t[j] = gacc[d][j] - cmu * acc[d][j] + pacc[d][j];
+            for (int j = 0; j < 16; ++j) t[j] = tacc[d][j] - cmu * acc[d][j];
             store_acc<T>(trow, 32 * d, hf, p.D, t, inv_l, vec);
         }
     }
+    SJVP_TS_DUMP(p.dbg, 0);
 }
 
 }  // namespace sjvp
