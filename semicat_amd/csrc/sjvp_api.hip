@@ -54,18 +54,23 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
     return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
 }
 
-// Ring depth (stages of 32 rows in flight) per head-dimension class.
+// Ring depths (stages of 32 rows in flight) per head-dimension class, sized to the LDS left beside
+// the workgroup's own rows (160 KB per CU; the forward keeps two workgroups per CU resident).
 template <int HD>
 struct Ring {
-    static constexpr int depth = HD == 128 ? 3 : 4;
+    static constexpr int fwd = HD == 128 ? 2 : 4;         // with tangents (four slabs per stage)
+    static constexpr int fwd_primal = 4;                  // primal only (two slabs per stage)
+    static constexpr int row = 3;
+    static constexpr int col = HD == 128 ? 3 : 4;
 };
 
 template <typename T, int HD, bool DMA>
 int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    constexpr int R = DMA ? Ring<HD>::depth : 1;
+    constexpr int R = DMA ? Ring<HD>::fwd : 1;
+    constexpr int RP = DMA ? Ring<HD>::fwd_primal : 1;
     if (jvp)
-        return launch(fwd_kernel<T, HD, R, true, DMA>, grid, FwdSmem<HD, R, true>::bytes, stream, p);
-    return launch(fwd_kernel<T, HD, R, false, DMA>, grid, FwdSmem<HD, R, false>::bytes, stream, p);
+        return launch(fwd_kernel<T, HD, R, true, DMA>, grid, FwdSmem<HD, R, true, DMA>::bytes, stream, p);
+    return launch(fwd_kernel<T, HD, RP, false, DMA>, grid, FwdSmem<HD, RP, false, DMA>::bytes, stream, p);
 }
 
 template <typename T>
@@ -83,31 +88,24 @@ int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
 
 template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
 int bwd_mode(const BwdParams& p, int BH, hipStream_t stream) {
-    constexpr int R = DMA ? Ring<HD>::depth : 1;
+    constexpr int R = DMA ? Ring<HD>::row : 1;
+    constexpr int CR = DMA ? Ring<HD>::col : 1;
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.
     int rc = launch(bwd_row_kernel<T, HD, R, HAS_DO, HAS_G, DMA>, BH * p.q_blocks,
-                    RowSmem<HD, R, HAS_G>::bytes, stream, p);
+                    RowSmem<HD, R, HAS_DO, HAS_G, DMA>::bytes, stream, p);
     if (rc != SJVP_OK) return rc;
     const int col_grid = BH * p.k_blocks;
-    using SM = ColSmem<HD, R, HAS_DO, HAS_G>;
+    using SM = ColSmem<HD, CR, HAS_DO, HAS_G, DMA>;
     if constexpr (HD == 128) {
         // two launches, each accumulating half of the head dimension (register budget)
-        rc = launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 0, 2, DMA>, col_grid, SM::bytes,
+        rc = launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 0, 2, DMA>, col_grid, SM::bytes,
                     stream, p);
         if (rc != SJVP_OK) return rc;
-        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 2, 2, DMA>, col_grid,
+        return launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 2, 2, DMA>, col_grid,
                       SM::bytes, stream, p);
     } else {
-#ifdef SJVP_X_SPLITCOL
-        rc = launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, false, 0, HD / 32, DMA>, col_grid,
-                    SM::bytes, stream, p);
-        if (rc != SJVP_OK) return rc;
-        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, false, true, 0, HD / 32, DMA>, col_grid,
+        return launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 0, HD / 32, DMA>, col_grid,
                       SM::bytes, stream, p);
-#else
-        return launch(bwd_col_kernel<T, HD, R, HAS_DO, HAS_G, true, true, 0, HD / 32, DMA>, col_grid,
-                      SM::bytes, stream, p);
-#endif
     }
 }
 
@@ -131,11 +129,6 @@ int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t s
 }
 
 }  // namespace
-
-#ifdef SJVP_X_TIMING
-static unsigned long long* g_dbg = nullptr;
-extern "C" void sjvp_x_set_debug(void* p) { g_dbg = static_cast<unsigned long long*>(p); }
-#endif
 
 extern "C" {
 
@@ -175,9 +168,6 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
-#ifdef SJVP_X_TIMING
-    p.dbg = g_dbg;
-#endif
     const int grid = B * H * p.q_blocks;
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == SJVP_BF16 ? fwd_dtype<Bf16>(p, grid, jvp, s) : fwd_dtype<Fp16>(p, grid, jvp, s);
@@ -247,9 +237,6 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
-#ifdef SJVP_X_TIMING
-    p.dbg = g_dbg;
-#endif
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, s)
                               : bwd_dtype<Fp16>(p, B * H, has_do, has_g, s);

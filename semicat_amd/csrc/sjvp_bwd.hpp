@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "sjvp_device.hpp"
+#include "sjvp_stream.hpp"
 
 namespace sjvp {
 
@@ -36,26 +37,37 @@ struct BwdParams {
     int q_blocks, k_blocks;  // ceil(L / 128)
     float scale;
     int vec;
-#ifdef SJVP_X_TIMING
-    unsigned long long* dbg;
-#endif
 };
 
 // ---------------------------------------------------------------------------------------------
 // Row-owned kernel: dQ (and dQ_dot).  Tiles are transposed (rows = keys in registers, columns =
 // this wave's queries in lanes), so the row statistics are per-lane scalars.
-template <int HD, int R, bool HAS_G>
+// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's 128 rows of Q, O (, Q_dot, G, TO)
+// (, dO), 4 slabs each][lse and mu of those rows][ring of K, V (, K_dot, V_dot) stages]; the ring
+// doubles as store staging after the last stage.
+template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
 struct RowSmem {
+    static constexpr bool own_lds = DMA && HD <= 64;
     static constexpr int nt = HAS_G ? 4 : 2;
     static constexpr int slot = nt * Slab<HD>::elems;
-    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
+    static constexpr int n_own = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
+    static constexpr int own = own_lds ? n_own * 4 * Slab<HD>::elems : 0;
+    static constexpr int stat = own_lds ? 2 * kOwned * 2 : 0;  // two float arrays, in elem_t units
+    static constexpr int bytes = (own + stat + R * slot) * (int)sizeof(elem_t);
 };
 
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
-__global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p) {
+__global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = RowSmem<HD, R, HAS_G>;
-    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    using SM = RowSmem<HD, R, HAS_DO, HAS_G, DMA>;
+    constexpr bool OWN_LDS = SM::own_lds;
+    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
+    float* own_stat = reinterpret_cast<float*>(own + SM::own);
+    elem_t* ring = own + SM::own + SM::stat;
+    // own tensor order: Q, O, [Q_dot, G, TO], [dO]
+    constexpr int oQ = 0, oO = 4 * Slab<HD>::elems, oTQ = 8 * Slab<HD>::elems,
+                  oG = 12 * Slab<HD>::elems, oTO = 16 * Slab<HD>::elems,
+                  oDO = (HAS_G ? 20 : 8) * Slab<HD>::elems;
 
     constexpr int KC = HD / 16;
     constexpr int DT = HD / 32;
@@ -69,25 +81,51 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p)
     const int qb = blockIdx.x % p.q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
-
-    SJVP_TS_DECL;
-    SJVP_TS(0);
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
 
-    u32x4 qB[KC], tqB[KC], gB[KC], doB[KC];
-    {
-        const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
+    u32x4 qB[KC], tqB[KC], gB[KC], doB[KC], oR[KC], toR[KC];
+    float lse2 = 0.f, mu = 0.f;
+    const int64_t so = (int64_t)bh * p.Lr + qrow;
+    if constexpr (OWN_LDS) {
+        // coalesced LDS-DMA copies of the workgroup's own rows; they are read back as B operands
+        // after the first ring stages have been issued
+        const int r0 = qb * kOwned;
+        auto own_fill = [&](int off, const TensorView& t) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c) qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
+            for (int s4 = 0; s4 < 4; ++s4)
+                fill_slab<HD, true>(own + off + s4 * Slab<HD>::elems, t.head(b, h), t.sl, r0 + 32 * s4,
+                                    p.Lq, p.D, true, tid);
+        };
+        own_fill(oQ, p.q);
+        own_fill(oO, p.o);
+        if constexpr (HAS_G) {
+            own_fill(oTQ, p.tq);
+            own_fill(oG, p.dTO);
+            own_fill(oTO, p.to);
+        }
+        if constexpr (HAS_DO) own_fill(oDO, p.dO);
+        // lse (lanes 0-31) and mu (lanes 32-63) of this wave's 32 rows; rows < Lr exist in both
+        const float* src = hf == 0 ? p.lse : p.mu;
+        if (HAS_G || hf == 0) dma4(src + so, lds_addr(own_stat) + (uint32_t)(wave * 64 * 4));
+    } else {
+        const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
+        const elem_t* op = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
+            oR[c] = load8(op, 16 * c + 8 * hf, p.D, qvalid, vec);
+        }
         if constexpr (HAS_G) {
             const elem_t* tqp = p.tq.head(b, h) + (int64_t)qrow * p.tq.sl;
             const elem_t* gp = p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl;
+            const elem_t* top = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
                 tqB[c] = load8(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
                 gB[c] = load8(gp, 16 * c + 8 * hf, p.D, qvalid, vec);
+                toR[c] = load8(top, 16 * c + 8 * hf, p.D, qvalid, vec);
             }
         }
         if constexpr (HAS_DO) {
@@ -95,31 +133,37 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p)
 #pragma unroll
             for (int c = 0; c < KC; ++c) doB[c] = load8(dop, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
+        // Per-lane row statistics; an invalid query lane uses zeros (finite P, results discarded).
+        lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
+        mu = (qvalid && HAS_G) ? p.mu[so] : 0.f;
+        if constexpr (DMA) {
+            // retire these loads before the first LDS-DMA copy so that wait_vmcnt() only has the
+            // ring's traffic to count
+            asm volatile("" : "+v"(lse2), "+v"(mu));
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                asm volatile("" : "+v"(qB[c]), "+v"(oR[c]));
+                if constexpr (HAS_G) asm volatile("" : "+v"(tqB[c]), "+v"(gB[c]), "+v"(toR[c]));
+                if constexpr (HAS_DO) asm volatile("" : "+v"(doB[c]));
+            }
+        }
     }
-    // Per-lane row statistics; an invalid query lane uses zeros (finite P, results discarded).
-    const int64_t so = (int64_t)bh * p.Lr + qrow;
-    const float lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
-    const float mu = (qvalid && HAS_G) ? p.mu[so] : 0.f;
+
     // s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O): each half-lane holds half of the row's
-    // columns of G and dO as B operands; O and TO are read in the same pattern.
+    // columns (those of its B operands); the two halves are added across the wave.
     float s4 = 0.f, s7d = 0.f;
-    {
-        const elem_t* op = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
-        const elem_t* top = HAS_G ? p.to.head(b, h) + (int64_t)qrow * p.to.sl : nullptr;
+    auto row_sums = [&]() {
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-            const u32x4 ov = load8(op, 16 * c + 8 * hf, p.D, qvalid, vec);
-            u32x4 tov;
-            if constexpr (HAS_G) tov = load8(top, 16 * c + 8 * hf, p.D, qvalid, vec);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float o0 = T::to_float((elem_t)(ov[i] & 0xffffu));
-                const float o1 = T::to_float((elem_t)(ov[i] >> 16));
+                const float o0 = T::to_float((elem_t)(oR[c][i] & 0xffffu));
+                const float o1 = T::to_float((elem_t)(oR[c][i] >> 16));
                 if constexpr (HAS_G) {
                     const float g0 = T::to_float((elem_t)(gB[c][i] & 0xffffu));
                     const float g1 = T::to_float((elem_t)(gB[c][i] >> 16));
-                    const float t0 = T::to_float((elem_t)(tov[i] & 0xffffu));
-                    const float t1 = T::to_float((elem_t)(tov[i] >> 16));
+                    const float t0 = T::to_float((elem_t)(toR[c][i] & 0xffffu));
+                    const float t1 = T::to_float((elem_t)(toR[c][i] >> 16));
                     s4 += g0 * o0 + g1 * o1;
                     s7d += g0 * t0 + g1 * t1;
                 }
@@ -132,28 +176,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p)
         }
         s4 += other_half(s4);
         s7d += other_half(s7d);
-        if (hf == 0) {  // every row below Lr is written (zeros beyond Lq): the column-owned
-                        // kernel, which runs after this one, stages whole 32-row groups
-            p.lse2[so] = lse2;
-            p.s4[so] = s4;
-            p.s7d[so] = s7d;
-        }
-    }
-    if constexpr (DMA) {
-        // Everything loaded so far has been consumed above except the B operands: retire them
-        // before the first LDS-DMA copy so that wait_vmcnt() only has the ring's traffic to count.
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
-            asm volatile("" : "+v"(qB[c]));
-            if constexpr (HAS_G) {
-                asm volatile("" : "+v"(tqB[c]));
-                asm volatile("" : "+v"(gB[c]));
-            }
-            if constexpr (HAS_DO) asm volatile("" : "+v"(doB[c]));
-        }
-    }
-
-    SJVP_TS(1);
+    };
+    if constexpr (!OWN_LDS) row_sums();
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = HAS_G ? p.tk.head(b, h) : nullptr;
@@ -237,15 +261,36 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p)
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
     if constexpr (DMA) {
-        for (int s = 0; s < R && s < n; ++s) issue(s);
+        int issued = 0;
+        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
+        if constexpr (OWN_LDS) {
+            wait_vmcnt(issued * SPT);  // the own rows were issued before these stages
+            __syncthreads();
+            const int sw = wave * Slab<HD>::elems;
+            read_b_operands<HD>(qB, own + oQ + sw, x, hf);
+            read_b_operands<HD>(oR, own + oO + sw, x, hf);
+            if constexpr (HAS_G) {
+                read_b_operands<HD>(tqB, own + oTQ + sw, x, hf);
+                read_b_operands<HD>(gB, own + oG + sw, x, hf);
+                read_b_operands<HD>(toR, own + oTO + sw, x, hf);
+            }
+            if constexpr (HAS_DO) read_b_operands<HD>(doB, own + oDO + sw, x, hf);
+            lse2 = own_stat[wave * 64 + x] * kLog2e;
+            if constexpr (HAS_G) mu = own_stat[wave * 64 + 32 + x];
+            row_sums();
+        }
     }
-    SJVP_TS(2);
+    if (hf == 0) {  // every row below Lr is written (zeros beyond Lq except lse2, which is finite):
+                    // the column-owned kernel, which runs after this one, stages 32-row groups
+        p.lse2[so] = lse2;
+        p.s4[so] = s4;
+        p.s7d[so] = s7d;
+    }
     for (int i = 0; i < n; ++i) {
         if constexpr (DMA) {
             wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
             __syncthreads();
             if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-            if (i == 0) { SJVP_TS(3); }
         } else {
             __syncthreads();
             issue(i);
@@ -260,30 +305,44 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_row_kernel(const BwdParams p)
             compute(slot, k0, std::false_type{});
         }
     }
-
-    SJVP_TS(4);
-    if (!qvalid) return;
-    elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
+    if constexpr (DMA) {
+        __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+        if (!wave_active) return;
+        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
+        const int row0 = qb * kOwned + wave * 32;
+        store_tile_coalesced<T, HD>(stage_tile, p.dq.head(b, h), p.dq.sl, row0, p.Lq, p.D, dq, p.scale,
+                                    lane);
+        if constexpr (HAS_G)
+            store_tile_coalesced<T, HD>(stage_tile, p.dtq.head(b, h), p.dtq.sl, row0, p.Lq, p.D, dtq,
+                                        p.scale, lane);
+    } else {
+        if (!qvalid) return;
+        elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
 #pragma unroll
-    for (int d = 0; d < DT; ++d) store_acc<T>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
-    if constexpr (HAS_G) {
-        elem_t* dtqrow = p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl;
+        for (int d = 0; d < DT; ++d) store_acc<T>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
+        if constexpr (HAS_G) {
+            elem_t* dtqrow = p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
+            for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
+        }
     }
-    SJVP_TS_DUMP(p.dbg, 1);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Column-owned kernel: a wavefront owns 32 keys and streams the queries.  DO_K selects dK (and
 // dK_dot), DO_V selects dV (and dV_dot); DT0/NDT select the 32-wide head-dimension tiles that are
 // accumulated (at HD = 128 the work is split to stay inside the register file).
-template <int HD, int R, bool HAS_DO, bool HAS_G>
+// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's 128 rows of K, V (, K_dot, V_dot),
+// 4 slabs each][ring of Q (, Q_dot, G) (, dO) stages, each followed by its row statistics]; the
+// ring doubles as store staging after the last stage.
+template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
 struct ColSmem {
+    static constexpr bool own_lds = DMA && HD <= 64;
     static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
     static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
     static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
-    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
+    static constexpr int own = own_lds ? (HAS_G ? 4 : 2) * 4 * Slab<HD>::elems : 0;
+    static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
 };
 
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT,
@@ -291,9 +350,11 @@ template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DO_K, bool DO
 __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd_col_kernel(
     const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = ColSmem<HD, R, HAS_DO, HAS_G>;
-    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
-    // slot layout: Q | [Q_dot | G] | [dO] | stats(lse2, mu, s4, s7d)
+    using SM = ColSmem<HD, R, HAS_DO, HAS_G, DMA>;
+    constexpr bool OWN_LDS = SM::own_lds;
+    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
+    elem_t* ring = own + SM::own;
+    // own tensor order: K, V, [K_dot, V_dot];  slot layout: Q | [Q_dot | G] | [dO] | stats(lse2, mu, s4, s7d)
     constexpr int oTQ = Slab<HD>::elems;
     constexpr int oG = 2 * Slab<HD>::elems;
     constexpr int oDO = (HAS_G ? 3 : 1) * Slab<HD>::elems;
@@ -312,15 +373,26 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     // LDS-DMA instructions per stage issued by this wave: the tensors, plus one 4-byte copy of two
     // statistic arrays by waves 0 and 1
     const int spt = SM::nt * Slab<HD>::per_thread + (wave < 2 ? 1 : 0);
-
-    SJVP_TS_DECL;
-    SJVP_TS(0);
     const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;
 
     u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    {
+    if constexpr (OWN_LDS) {
+        const int r0 = kb * kOwned;
+        auto own_fill = [&](int idx, const TensorView& t) {
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4)
+                fill_slab<HD, true>(own + (4 * idx + s4) * Slab<HD>::elems, t.head(b, h), t.sl,
+                                    r0 + 32 * s4, p.Lk, p.D, true, tid);
+        };
+        own_fill(0, p.k);
+        own_fill(1, p.v);
+        if constexpr (HAS_G) {
+            own_fill(2, p.tk);
+            own_fill(3, p.tv);
+        }
+    } else {
         const elem_t* kp = p.k.head(b, h) + (int64_t)krow * p.k.sl;
         const elem_t* vp = p.v.head(b, h) + (int64_t)krow * p.v.sl;
 #pragma unroll
@@ -349,8 +421,6 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
             }
         }
     }
-
-    SJVP_TS(1);
     const elem_t* qg = p.q.head(b, h);
     const elem_t* tqg = HAS_G ? p.tq.head(b, h) : nullptr;
     const elem_t* gg = HAS_G ? p.dTO.head(b, h) : nullptr;
@@ -483,15 +553,24 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
 
     const int n = (p.Lq + kStageRows - 1) / kStageRows;
     if constexpr (DMA) {
-        for (int s = 0; s < R && s < n; ++s) issue(s);
+        int issued = 0;
+        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
+        if constexpr (OWN_LDS) {
+            wait_vmcnt(issued * spt);  // the own rows were issued before these stages
+            __syncthreads();
+            read_b_operands<HD>(kB, own + wave * Slab<HD>::elems, x, hf);
+            if constexpr (DO_K) read_b_operands<HD>(vB, own + (4 + wave) * Slab<HD>::elems, x, hf);
+            if constexpr (HAS_G) {
+                read_b_operands<HD>(tkB, own + (8 + wave) * Slab<HD>::elems, x, hf);
+                if constexpr (DO_K) read_b_operands<HD>(tvB, own + (12 + wave) * Slab<HD>::elems, x, hf);
+            }
+        }
     }
-    SJVP_TS(2);
     for (int i = 0; i < n; ++i) {
         if constexpr (DMA) {
             wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * spt);
             __syncthreads();
             if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-            if (i == 0) { SJVP_TS(3); }
         } else {
             __syncthreads();
             issue(i);
@@ -500,33 +579,53 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
         if (!wave_active) continue;
         compute(ring + (i % R) * SM::slot);
     }
-
-    SJVP_TS(4);
-    if (!kvalid) return;
-    if constexpr (DO_K) {
-        elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;
-#pragma unroll
-        for (int d = 0; d < NDT; ++d)
-            store_acc<T>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
-        if constexpr (HAS_G) {
-            elem_t* dtkrow = p.dtk.head(b, h) + (int64_t)krow * p.dtk.sl;
+    if constexpr (DMA) {
+        __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+        if (!wave_active) return;
+        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
+        const int row0 = kb * kOwned + wave * 32;
+        // NDT tiles starting at head-dimension tile DT0: the staging tile and the row pointers are
+        // offset by 32*DT0 columns, and the column bound is reduced accordingly
+        const int dcol = 32 * DT0;
+        auto put = [&](const OutView& t, const f32x16* acc, float mul) {
+            store_tile_coalesced<T, 32 * NDT>(stage_tile, t.head(b, h) + dcol, t.sl, row0, p.Lk,
+                                              p.D - dcol, acc, mul, lane);
+        };
+        if constexpr (DO_K) {
+            put(p.dk, dk, p.scale);
+            if constexpr (HAS_G) put(p.dtk, dtk, p.scale);
+        }
+        if constexpr (DO_V) {
+            put(p.dv, dv, 1.0f);
+            if constexpr (HAS_G) put(p.dtv, dtv, 1.0f);
+        }
+    } else {
+        if (!kvalid) return;
+        if constexpr (DO_K) {
+            elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;
 #pragma unroll
             for (int d = 0; d < NDT; ++d)
-                store_acc<T>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
-        }
-    }
-    if constexpr (DO_V) {
-        elem_t* dvrow = p.dv.head(b, h) + (int64_t)krow * p.dv.sl;
+                store_acc<T>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
+            if constexpr (HAS_G) {
+                elem_t* dtkrow = p.dtk.head(b, h) + (int64_t)krow * p.dtk.sl;
 #pragma unroll
-        for (int d = 0; d < NDT; ++d) store_acc<T>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
-        if constexpr (HAS_G) {
-            elem_t* dtvrow = p.dtv.head(b, h) + (int64_t)krow * p.dtv.sl;
+                for (int d = 0; d < NDT; ++d)
+                    store_acc<T>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
+            }
+        }
+        if constexpr (DO_V) {
+            elem_t* dvrow = p.dv.head(b, h) + (int64_t)krow * p.dv.sl;
 #pragma unroll
             for (int d = 0; d < NDT; ++d)
-                store_acc<T>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
+                store_acc<T>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
+            if constexpr (HAS_G) {
+                elem_t* dtvrow = p.dtv.head(b, h) + (int64_t)krow * p.dtv.sl;
+#pragma unroll
+                for (int d = 0; d < NDT; ++d)
+                    store_acc<T>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
+            }
         }
     }
-    SJVP_TS_DUMP(p.dbg, 2);
 }
 
 }  // namespace sjvp

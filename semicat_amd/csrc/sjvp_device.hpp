@@ -29,24 +29,6 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#ifdef SJVP_X_TIMING
-#define SJVP_TS_DECL unsigned long long tstamp[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define SJVP_TS(i) tstamp[i] = __builtin_readcyclecounter()
-#define SJVP_TS_DUMP(dbg, kid)                                                              \
-    do {                                                                                    \
-        __builtin_amdgcn_s_waitcnt(0);                                                      \
-        SJVP_TS(5);                                                                         \
-        if ((threadIdx.x & 63) == 0 && (dbg)) {                                             \
-            unsigned long long* d_ = (dbg) + ((size_t)(kid) * 4096 + blockIdx.x * 4 + (threadIdx.x >> 6)) * 8; \
-            for (int i_ = 0; i_ < 6; ++i_) d_[i_] = tstamp[i_];                             \
-        }                                                                                   \
-    } while (0)
-#else
-#define SJVP_TS_DECL
-#define SJVP_TS(i)
-#define SJVP_TS_DUMP(dbg, kid)
-#endif
-
 namespace sjvp {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -168,19 +150,20 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 
 // LDS-DMA: each active lane copies 16 bytes from its global address to LDS byte address
-// base + 16 * lane_id (base must be wave-uniform).  Completion is tracked by vmcnt only.
+// base + 16 * lane_id (base must be wave-uniform).  Completion is tracked by vmcnt only.  M0 carries
+// the LDS base; nothing else in these kernels uses M0 (gfx9 LDS instructions do not need it).
 __device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
+                 : "memory");
 }
 // 4-byte form: LDS byte address base + 4 * lane_id.
 __device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off"
                  :
                  : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_base))
-                 : "memory", "m0");
+                 : "memory");
 }
 
 // s_waitcnt vmcnt(n) for a run-time n (clamped to the encodable 0..63): at most n of this wave's

@@ -11,6 +11,7 @@
 #include <type_traits>
 
 #include "sjvp_device.hpp"
+#include "sjvp_stream.hpp"
 
 namespace sjvp {
 
@@ -24,16 +25,18 @@ struct FwdParams {
     int q_blocks;  // ceil(Lq / 128)
     float scale;
     int vec;  // all tensors 16-byte aligned, strides % 8 == 0, D % 8 == 0
-#ifdef SJVP_X_TIMING
-    unsigned long long* dbg;
-#endif
 };
 
-template <int HD, int R, bool JVP>
+// LDS layout: [own: Q (and Q_dot) rows of the workgroup, 4 slabs each - LDS-DMA path only]
+//             [ring: R slots of K, V (, K_dot, V_dot) stage slabs]
+// After the last stage the ring memory doubles as the per-wave staging tiles of the output stores.
+template <int HD, int R, bool JVP, bool DMA>
 struct FwdSmem {
     static constexpr int nt = JVP ? 4 : 2;                      // tensors per stage
     static constexpr int slot = nt * Slab<HD>::elems;            // elements per ring slot
-    static constexpr int bytes = R * slot * (int)sizeof(elem_t);
+    static constexpr int own = DMA ? (JVP ? 2 : 1) * 4 * Slab<HD>::elems : 0;
+    static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
+    static_assert(!DMA || R * slot >= kWaves * StoreStage<HD>::elems, "ring too small to stage stores");
 };
 
 // The reference maximum of the online softmax is only raised when a new tile exceeds it by more
@@ -43,10 +46,11 @@ struct FwdSmem {
 constexpr float kMaxSlack = 6.0f;
 
 template <typename T, int HD, int R, bool JVP, bool DMA>
-__global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = FwdSmem<HD, R, JVP>;
-    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    using SM = FwdSmem<HD, R, JVP, DMA>;
+    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
+    elem_t* ring = own + SM::own;
 
     constexpr int KC = HD / 16;  // k-chunks of the score contraction
     constexpr int DT = HD / 32;  // 32-wide tiles of the head dimension
@@ -62,16 +66,25 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
     const int qb = blockIdx.x % p.q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
-
-    SJVP_TS_DECL;
-    SJVP_TS(0);
     const int qrow = qb * kOwned + wave * 32 + x;  // the query this lane owns
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
 
-    // Owned-side operands (B of S^T = K Q^T), kept in registers for the whole pass.
+    // Owned-side operands (B of S^T = K Q^T), kept in registers for the whole pass.  On the LDS-DMA
+    // path they are copied coalesced into LDS first (issued here, read after the first stages have
+    // been issued); otherwise every lane loads its own row.
     u32x4 qB[KC], tqB[KC];
-    {
+    if constexpr (DMA) {
+        const int r0 = qb * kOwned;
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+            fill_slab<HD, true>(own + s4 * Slab<HD>::elems, p.q.head(b, h), p.q.sl, r0 + 32 * s4, p.Lq,
+                                p.D, true, tid);
+            if constexpr (JVP)
+                fill_slab<HD, true>(own + (4 + s4) * Slab<HD>::elems, p.tq.head(b, h), p.tq.sl,
+                                    r0 + 32 * s4, p.Lq, p.D, true, tid);
+        }
+    } else {
         const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
 #pragma unroll
         for (int c = 0; c < KC; ++c) qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
@@ -80,18 +93,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int c = 0; c < KC; ++c) tqB[c] = load8(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
-        if constexpr (DMA) {
-            // Retire these loads before the first LDS-DMA copy is issued: afterwards the only
-            // vector-memory traffic in flight is the ring's, which wait_vmcnt() counts.
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                asm volatile("" : "+v"(qB[c]));
-                if constexpr (JVP) asm volatile("" : "+v"(tqB[c]));
-            }
-        }
     }
-
-    SJVP_TS(1);
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = JVP ? p.tk.head(b, h) : nullptr;
@@ -123,33 +125,46 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
         if constexpr (JVP) tacc[t] = f32x16{0};
     }
 
-    auto compute = [&](const elem_t* slot, int k0, auto ragged_tag) {
+    // One online-softmax step over NS consecutive stages (slots slot0, slot1): the score tiles of
+    // all NS stages are formed first, so that their MFMA chains, the exponentials and the output
+    // contractions of different stages overlap inside the wave.  Only the last stage of the step
+    // can be ragged.
+    auto compute = [&](const elem_t* slot0, const elem_t* slot1, int k0, auto ns_tag, auto ragged_tag) {
+        constexpr int NS = decltype(ns_tag)::value;
         constexpr bool RAGGED = decltype(ragged_tag)::value;
-        const elem_t* sK = slot;
-        const elem_t* sV = slot + Slab<HD>::elems;
-        const elem_t* sTK = slot + 2 * Slab<HD>::elems;
-        const elem_t* sTV = slot + 3 * Slab<HD>::elems;
-        f32x16 s = {0}, ts = {0};
+        const elem_t* slots[2] = {slot0, slot1};
+        f32x16 s[NS], ts[NS];
+#pragma unroll
+        for (int g = 0; g < NS; ++g) {
+            s[g] = f32x16{0};
+            ts[g] = f32x16{0};
+        }
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-            u32x4 a = lds_a_rows<HD>(sK, c, x, hf);
-            s = T::mfma(a, qB[c], s);
-            if constexpr (JVP) {
-                ts = T::mfma(a, tqB[c], ts);
-                u32x4 at = lds_a_rows<HD>(sTK, c, x, hf);
-                ts = T::mfma(at, qB[c], ts);
+#pragma unroll
+            for (int g = 0; g < NS; ++g) {
+                u32x4 a = lds_a_rows<HD>(slots[g], c, x, hf);
+                s[g] = T::mfma(a, qB[c], s[g]);
+                if constexpr (JVP) {
+                    ts[g] = T::mfma(a, tqB[c], ts[g]);
+                    u32x4 at = lds_a_rows<HD>(slots[g] + 2 * Slab<HD>::elems, c, x, hf);
+                    ts[g] = T::mfma(at, qB[c], ts[g]);
+                }
             }
         }
         if constexpr (RAGGED) {
             // keys beyond Lk are zero rows in LDS (their S_dot is already 0)
+            const int kl = k0 + (NS - 1) * kStageRows;
 #pragma unroll
             for (int j = 0; j < 16; ++j)
-                if (k0 + 8 * (j >> 2) + 4 * hf + (j & 3) >= p.Lk) s[j] = -INFINITY;
+                if (kl + 8 * (j >> 2) + 4 * hf + (j & 3) >= p.Lk) s[NS - 1][j] = -INFINITY;
         }
-        float mloc = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+        float mloc = -INFINITY;
 #pragma unroll
-        for (int j = 4; j < 16; j += 4)
-            mloc = fmaxf(mloc, fmaxf(fmaxf(s[j], s[j + 1]), fmaxf(s[j + 2], s[j + 3])));
+        for (int g = 0; g < NS; ++g)
+#pragma unroll
+            for (int j = 0; j < 16; j += 4)
+                mloc = fmaxf(mloc, fmaxf(fmaxf(s[g][j], s[g][j + 1]), fmaxf(s[g][j + 2], s[g][j + 3])));
         mloc = fmaxf(mloc, other_half(mloc)) * sl2;
         m_true = fmaxf(m_true, mloc);
         if (__builtin_amdgcn_ballot_w64(mloc > m_i + kMaxSlack) != 0) {  // wave-uniform branch
@@ -166,31 +181,39 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
         }
         float lsum = 0.f, musum = 0.f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const float pj = fast_exp2(fmaf(s[j], sl2, -m_i));
-            s[j] = pj;
-            lsum += pj;
-            if constexpr (JVP) {
-                const float pt = pj * (ts[j] * p.scale);
-                ts[j] = pt;
-                musum += pt;
+        for (int g = 0; g < NS; ++g) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const float pj = fast_exp2(fmaf(s[g][j], sl2, -m_i));
+                s[g][j] = pj;
+                lsum += pj;
+                if constexpr (JVP) {
+                    const float pt = pj * (ts[g][j] * p.scale);
+                    ts[g][j] = pt;
+                    musum += pt;
+                }
             }
         }
         l_i += lsum;
         if constexpr (JVP) mu_i += musum;
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            u32x4 pb = pack_b<T>(s, c);
-            u32x4 ptb;
-            if constexpr (JVP) ptb = pack_b<T>(ts, c);
 #pragma unroll
-            for (int d = 0; d < DT; ++d) {
-                u32x4 av = lds_a_transposed<HD>(sV, c, 32 * d, lane);
-                acc[d] = T::mfma(av, pb, acc[d]);
-                if constexpr (JVP) {
-                    tacc[d] = T::mfma(av, ptb, tacc[d]);
-                    u32x4 atv = lds_a_transposed<HD>(sTV, c, 32 * d, lane);
-                    tacc[d] = T::mfma(atv, pb, tacc[d]);
+            for (int g = 0; g < NS; ++g) {
+                const elem_t* sV = slots[g] + Slab<HD>::elems;
+                const elem_t* sTV = slots[g] + 3 * Slab<HD>::elems;
+                u32x4 pb = pack_b<T>(s[g], c);
+                u32x4 ptb;
+                if constexpr (JVP) ptb = pack_b<T>(ts[g], c);
+#pragma unroll
+                for (int d = 0; d < DT; ++d) {
+                    u32x4 av = lds_a_transposed<HD>(sV, c, 32 * d, lane);
+                    acc[d] = T::mfma(av, pb, acc[d]);
+                    if constexpr (JVP) {
+                        tacc[d] = T::mfma(av, ptb, tacc[d]);
+                        u32x4 atv = lds_a_transposed<HD>(sTV, c, 32 * d, lane);
+                        tacc[d] = T::mfma(atv, pb, tacc[d]);
+                    }
                 }
             }
         }
@@ -198,31 +221,59 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
     if constexpr (DMA) {
-        for (int s = 0; s < R && s < n; ++s) issue(s);
+        int issued = 0;
+        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
+        // the owned rows were issued before these stages: they have landed once at most the
+        // stages' copies are outstanding
+        wait_vmcnt(issued * SPT);
+        __syncthreads();
+        read_b_operands<HD>(qB, own + wave * Slab<HD>::elems, x, hf);
+        if constexpr (JVP) read_b_operands<HD>(tqB, own + (4 + wave) * Slab<HD>::elems, x, hf);
     }
-    SJVP_TS(2);
-    for (int i = 0; i < n; ++i) {
-        if constexpr (DMA) {
-            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
-            __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
-            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-            if (i == 0) { SJVP_TS(3); }
-        } else {
-            __syncthreads();
-            issue(i);
-            __syncthreads();
+    using one_t = std::integral_constant<int, 1>;
+    using two_t = std::integral_constant<int, 2>;
+    if constexpr (DMA && R >= 3) {
+        // two stages per step: stage i+1 must have landed as well, and the slot of stage i-1 (and
+        // i-2) is refilled afterwards
+        int next = (R < n) ? R : n;  // next stage to issue
+        for (int i = 0, last = 0; i < n; i = last + 1) {
+            // pair up with stage i+1 only if it has been issued already
+            last = (i + 1 < next) ? i + 1 : i;
+            wait_vmcnt((next - 1 - last) * SPT);
+            __syncthreads();  // stages i..last have landed for every wave; stages < i are consumed
+            while (next < n && next < i + R) issue(next++);
+            if (!wave_active) continue;
+            const elem_t* s0 = ring + (i % R) * SM::slot;
+            const elem_t* s1 = ring + (last % R) * SM::slot;
+            const int k0 = i * kStageRows;
+            const bool ragged = (last + 1) * kStageRows > p.Lk;
+            if (last == i) {
+                if (ragged) compute(s0, s0, k0, one_t{}, std::true_type{});
+                else compute(s0, s0, k0, one_t{}, std::false_type{});
+            } else {
+                if (ragged) compute(s0, s1, k0, two_t{}, std::true_type{});
+                else compute(s0, s1, k0, two_t{}, std::false_type{});
+            }
         }
-        if (!wave_active) continue;
-        const elem_t* slot = ring + (i % R) * SM::slot;
-        const int k0 = i * kStageRows;
-        if (k0 + kStageRows > p.Lk) {
-            compute(slot, k0, std::true_type{});
-        } else {
-            compute(slot, k0, std::false_type{});
+    } else {
+        for (int i = 0; i < n; ++i) {
+            if constexpr (DMA) {
+                wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
+                __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+                if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
+            } else {
+                __syncthreads();
+                issue(i);
+                __syncthreads();
+            }
+            if (!wave_active) continue;
+            const elem_t* slot = ring + (i % R) * SM::slot;
+            const int k0 = i * kStageRows;
+            if (k0 + kStageRows > p.Lk) compute(slot, slot, k0, one_t{}, std::true_type{});
+            else compute(slot, slot, k0, one_t{}, std::false_type{});
         }
     }
-
-    SJVP_TS(4);
+    if constexpr (DMA) __syncthreads();  // every wave is done reading the ring
     if (!wave_active) {
         // All 32 rows of this wave lie beyond Lq: their statistic rows get the values a zero
         // query row produces (and the reference initialises them with): log(Lk), 0, Lk.
@@ -251,24 +302,34 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(const FwdParams p) {
         // to m_i, which may lag behind it by up to kMaxSlack.
         if (p.li) p.li[so] = l * fast_exp2(m_i - m_true);
     }
-    if (!qvalid) return;
-
-    elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
-#pragma unroll
-    for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
+    const float cmu = mu_un * inv_l;
     if constexpr (JVP) {
-        // TO = (g_acc - mu_un * O + p_tv_acc) / l     (ryu_triton.py:274-275)
-        elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
-        const float cmu = mu_un * inv_l;
+        // TO = (g_acc + p_tv_acc - mu_un * O) / l     (ryu_triton.py:274-275)
 #pragma unroll
-        for (int d = 0; d < DT; ++d) {
-            f32x16 t;
+        for (int d = 0; d < DT; ++d)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) t[j] = tacc[d][j] - cmu * acc[d][j];
-            store_acc<T>(trow, 32 * d, hf, p.D, t, inv_l, vec);
+            for (int j = 0; j < 16; ++j) tacc[d][j] -= cmu * acc[d][j];
+    }
+    if constexpr (DMA) {
+        // every wave of the workgroup reaches this point (inactive ones returned above only after
+        // the loop): the ring is free and becomes the staging area of coalesced row stores
+        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
+        const int row0 = qb * kOwned + wave * 32;
+        store_tile_coalesced<T, HD>(stage_tile, p.o.head(b, h), p.o.sl, row0, p.Lq, p.D, acc, inv_l, lane);
+        if constexpr (JVP)
+            store_tile_coalesced<T, HD>(stage_tile, p.to.head(b, h), p.to.sl, row0, p.Lq, p.D, tacc,
+                                        inv_l, lane);
+    } else {
+        if (!qvalid) return;
+        elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
+        if constexpr (JVP) {
+            elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) store_acc<T>(trow, 32 * d, hf, p.D, tacc[d], inv_l, vec);
         }
     }
-    SJVP_TS_DUMP(p.dbg, 0);
 }
 
 }  // namespace sjvp
