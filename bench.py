@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention-JVP forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu-baseline] [--calib-copy]
 
 A step is one pass of the hot path over one batch: the fused forward (O, TO, lse, mu) followed by
 the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
@@ -29,6 +29,13 @@ PRIMAL_SCALE, TANGENT_SCALE, SEED = 0.5, 0.1, 0
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
+# kernel of --calib-copy).  Commands and raw figures: profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "fwd_kernel": (2 * 37004.0 + 25344.0) * 1024,      # FETCH_SIZE counts 2 KiB per unit on the copy
+    "bwd_row_kernel": (2 * 61983.0 + 25728.0) * 1024,  # kernel (131089 for 262144 KiB), WRITE_SIZE 1 KiB
+    "bwd_col_kernel": (2 * 50090.5 + 49152.0) * 1024,
+}
 
 
 def step_flops(b=B, h=H, l=L, d=D) -> float:
@@ -84,6 +91,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a 256 MiB device copy (reference point for rocprofv3 --pmc byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (no multi-GPU path exists: "
@@ -106,11 +115,15 @@ def main() -> int:
     mu = torch.empty_like(lse)
     grads = tuple(torch.empty_like(q) for _ in range(6))
 
+    nbytes = _lib.load().sjvp_bwd_workspace_bytes(B, H, L, L, D, _lib.SJVP_BF16)
+    workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
+
     def fwd():
         kernels.attention_jvp_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False)
 
-    def bwd():
-        kernels.attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads)
+    def bwd(parts=_lib.SJVP_BWD_ALL):
+        kernels.attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads,
+                                       workspace=workspace, parts=parts)
 
     def step():
         fwd()
@@ -139,9 +152,10 @@ def main() -> int:
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
 
-        # per-phase durations with events on the launch stream (separate region, eager launches)
-        def timed(fn, n=50):
-            for _ in range(5):
+        # Per-kernel durations: HIP events on the launch stream around runs of one kernel launched
+        # alone (eager launches; every kernel sees the same buffers as in the timed steps).
+        def timed(fn, n=100):
+            for _ in range(10):
                 fn()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -152,31 +166,52 @@ def main() -> int:
             return e0.elapsed_time(e1) / n  # ms
 
         fwd_ms = timed(fwd)
+        row_ms = timed(lambda: bwd(_lib.SJVP_BWD_ROW))
+        col_ms = timed(lambda: bwd(_lib.SJVP_BWD_COL))
         bwd_ms = timed(bwd)
+
+        if a.calib_copy:
+            # a plain copy of known size, for scaling the FETCH_SIZE / WRITE_SIZE hardware counters
+            src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            stream.synchronize()
 
     ms_per_step = wall / a.steps * 1e3
     tflops = step_flops() / (ms_per_step * 1e-3) / 1e12
 
-    # Roofline of the forward kernel (one launch = the whole fused forward): algorithmic flops
-    # 12*L^2*D and bytes 8*L*D*2 (+12*L of statistics) per (batch, head).
-    fwd_flops = 12.0 * B * H * L * L * D
-    fwd_bytes = B * H * (8.0 * L * D * 2 + 12.0 * L)
-    bwd_flops = 30.0 * B * H * L * L * D
-    bwd_bytes = B * H * (16.0 * L * D * 2 + 16.0 * L)
-    # the backward launches dominate the step; its algorithmic intensity (flop/B) decides the bound
-    ai = bwd_flops / bwd_bytes
+    # Algorithmic work per (batch, head), e = 2 bytes.  The backward's 15 contractions and 16 tensor
+    # passes are credited once: the column-owned launch gets the 6 recomputed score-side contractions
+    # and its 6 output contractions (24 L^2 D flop) and the 8 tensors it reads plus the 4 it writes;
+    # the row-owned launch gets its 3 output contractions (6 L^2 D) and O, TO, dQ, dQ_dot (its second
+    # score-side pass and its re-read of the other eight inputs are redundant work, not credited).
+    BH = B * H
+    work = {
+        "fwd_kernel": {"ms": fwd_ms, "flops": 12.0 * BH * L * L * D, "bytes": BH * (8.0 * L * D * 2 + 8.0 * L)},
+        "bwd_row_kernel": {"ms": row_ms, "flops": 6.0 * BH * L * L * D, "bytes": BH * (4.0 * L * D * 2 + 12.0 * L)},
+        "bwd_col_kernel": {"ms": col_ms, "flops": 24.0 * BH * L * L * D, "bytes": BH * (12.0 * L * D * 2 + 16.0 * L)},
+    }
+    for w in work.values():
+        w["GBps"] = w["bytes"] / (w["ms"] * 1e-3) / 1e9
+        w["TFLOPs"] = w["flops"] / (w["ms"] * 1e-3) / 1e12
+    dom = max(work, key=lambda n: work[n]["ms"])
+    dk = work[dom]
     ridge = PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)
-    if ai < ridge:
-        achieved = bwd_bytes / (bwd_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                    "frac": achieved / PEAK_HBM_GBPS, "traffic": None}
+    if dk["flops"] / dk["bytes"] < ridge:
+        roofline = {"bound": "hbm", "achieved": dk["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": dk["GBps"] / PEAK_HBM_GBPS}
     else:
-        achieved = bwd_flops / (bwd_ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None}
-    roofline["kernel"] = "sjvp_bwd (rowstats + col + row launches)"
-    roofline["ms"] = bwd_ms
-    roofline["mfma_frac"] = bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS
+        roofline = {"bound": "mfma", "achieved": dk["TFLOPs"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": dk["TFLOPs"] / PEAK_BF16_TFLOPS}
+    # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+    # this script (scaled by the same counters on the --calib-copy kernel); see profiles/.
+    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom)
+    roofline["kernel"] = dom
+    roofline["ms"] = dk["ms"]
+    roofline["algorithmic_bytes"] = dk["bytes"]
+    roofline["algorithmic_flops"] = dk["flops"]
+    roofline["flop_per_byte"] = dk["flops"] / dk["bytes"]
 
     out = {
         "metric": METRIC,
@@ -198,8 +233,7 @@ def main() -> int:
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
-        "fwd_tflops": fwd_flops / (fwd_ms * 1e-3) / 1e12,
-        "fwd_gbps": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+        "kernels": {n: {"ms": w["ms"], "GBps": w["GBps"], "TFLOPs": w["TFLOPs"]} for n, w in work.items()},
         "roofline": roofline,
         "device": torch.cuda.get_device_name(0),
     }

@@ -50,7 +50,8 @@ enum sjvp_status {
     SJVP_ERR_DTYPE = -4,     /* dtype is neither SJVP_BF16 nor SJVP_FP16                     */
     SJVP_ERR_WORKSPACE = -5, /* workspace NULL or smaller than sjvp_bwd_workspace_bytes()    */
     SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (hipGetLastError)           */
-    SJVP_ERR_COTANGENT = -7  /* sjvp_bwd called with both dO and dTO NULL                    */
+    SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
+    SJVP_ERR_PARTS = -8      /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
 };
 
 /* Indices into the stride tables: strides[3*i + {0,1,2}] = (batch, head, sequence) strides in
@@ -86,9 +87,25 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
              void* dtv, void* workspace, size_t workspace_bytes, int B, int H, int Lq, int Lk, int D,
              const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
 
-/* Bytes of caller-provided device scratch sjvp_bwd needs (lse in log2 units and the row sums sum_4 and
- * sum_7 + delta, which
- * the reference allocates itself at flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
+/*
+ * The backward is two kernel launches: the row-owned one (dq, dtq, and the row sums it leaves in
+ * the workspace) and the column-owned one (dk, dv, dtk, dtv), which consumes that workspace.
+ * sjvp_bwd_parts() launches the selected ones with sjvp_bwd()'s arguments; sjvp_bwd() is
+ * sjvp_bwd_parts(SJVP_BWD_ALL, ...).  It has no counterpart in the reference: it exists so that a
+ * profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only valid on a
+ * workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.
+ */
+enum sjvp_bwd_part { SJVP_BWD_ROW = 1, SJVP_BWD_COL = 2, SJVP_BWD_ALL = 3 };
+int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const void* tq,
+                   const void* tk, const void* tv, const void* o, const void* to, const void* dO,
+                   const void* dTO, const float* lse, const float* mu, void* dq, void* dk, void* dv,
+                   void* dtq, void* dtk, void* dtv, void* workspace, size_t workspace_bytes, int B,
+                   int H, int Lq, int Lk, int D, const int64_t* strides /* [SJVP_B_COUNT*3] */,
+                   float scale, int dtype, void* stream);
+
+/* Bytes of caller-provided device scratch sjvp_bwd needs: lse in log2 units and the row sums sum_4
+ * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,
+ * flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
 
 /* Static, NUL-terminated description of a status code. */

@@ -19,12 +19,18 @@ SJVP_ERR_DTYPE = -4
 SJVP_ERR_WORKSPACE = -5
 SJVP_ERR_LAUNCH = -6
 SJVP_ERR_COTANGENT = -7
+SJVP_ERR_PARTS = -8
+
+SJVP_BWD_ROW = 1
+SJVP_BWD_COL = 2
+SJVP_BWD_ALL = 3
 
 F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
 B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
-EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_workspace_bytes", "sjvp_strerror", "sjvp_version")
+EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_workspace_bytes", "sjvp_strerror",
+           "sjvp_version")
 
 _lock = threading.Lock()
 _lib = None
@@ -54,6 +60,8 @@ def load() -> ctypes.CDLL:
             lib.sjvp_bwd.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [vp, ctypes.c_size_t] + [i] * 5 +
                                      [i64p, ctypes.c_float, i, vp])
             lib.sjvp_bwd.restype = i
+            lib.sjvp_bwd_parts.argtypes = [i] + lib.sjvp_bwd.argtypes
+            lib.sjvp_bwd_parts.restype = i
             lib.sjvp_bwd_workspace_bytes.argtypes = [i] * 6
             lib.sjvp_bwd_workspace_bytes.restype = ctypes.c_size_t
             lib.sjvp_strerror.argtypes = [i]

@@ -87,13 +87,15 @@ int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
 }
 
 template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
-int bwd_mode(const BwdParams& p, int BH, hipStream_t stream) {
+int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     constexpr int R = DMA ? Ring<HD>::row : 1;
     constexpr int CR = DMA ? Ring<HD>::col : 1;
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.
-    int rc = launch(bwd_row_kernel<T, HD, R, HAS_DO, HAS_G, DMA>, BH * p.q_blocks,
+    int rc = SJVP_OK;
+    if (parts & SJVP_BWD_ROW)
+        rc = launch(bwd_row_kernel<T, HD, R, HAS_DO, HAS_G, DMA>, BH * p.q_blocks,
                     RowSmem<HD, R, HAS_DO, HAS_G, DMA>::bytes, stream, p);
-    if (rc != SJVP_OK) return rc;
+    if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
     const int col_grid = BH * p.k_blocks;
     using SM = ColSmem<HD, CR, HAS_DO, HAS_G, DMA>;
     if constexpr (HD == 128) {
@@ -110,22 +112,22 @@ int bwd_mode(const BwdParams& p, int BH, hipStream_t stream) {
 }
 
 template <typename T, int HD, bool DMA>
-int bwd_hd(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
-    if (has_do && has_g) return bwd_mode<T, HD, true, true, DMA>(p, BH, stream);
-    if (has_g) return bwd_mode<T, HD, false, true, DMA>(p, BH, stream);
-    return bwd_mode<T, HD, true, false, DMA>(p, BH, stream);
+int bwd_hd(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
+    if (has_do && has_g) return bwd_mode<T, HD, true, true, DMA>(p, BH, parts, stream);
+    if (has_g) return bwd_mode<T, HD, false, true, DMA>(p, BH, parts, stream);
+    return bwd_mode<T, HD, true, false, DMA>(p, BH, parts, stream);
 }
 
 template <typename T>
-int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream) {
+int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
     if (p.vec) {
-        if (p.D <= 32) return bwd_hd<T, 32, true>(p, BH, has_do, has_g, stream);
-        if (p.D <= 64) return bwd_hd<T, 64, true>(p, BH, has_do, has_g, stream);
-        return bwd_hd<T, 128, true>(p, BH, has_do, has_g, stream);
+        if (p.D <= 32) return bwd_hd<T, 32, true>(p, BH, has_do, has_g, parts, stream);
+        if (p.D <= 64) return bwd_hd<T, 64, true>(p, BH, has_do, has_g, parts, stream);
+        return bwd_hd<T, 128, true>(p, BH, has_do, has_g, parts, stream);
     }
-    if (p.D <= 32) return bwd_hd<T, 32, false>(p, BH, has_do, has_g, stream);
-    if (p.D <= 64) return bwd_hd<T, 64, false>(p, BH, has_do, has_g, stream);
-    return bwd_hd<T, 128, false>(p, BH, has_do, has_g, stream);
+    if (p.D <= 32) return bwd_hd<T, 32, false>(p, BH, has_do, has_g, parts, stream);
+    if (p.D <= 64) return bwd_hd<T, 64, false>(p, BH, has_do, has_g, parts, stream);
+    return bwd_hd<T, 128, false>(p, BH, has_do, has_g, parts, stream);
 }
 
 }  // namespace
@@ -186,6 +188,17 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
              const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq, void* dtk,
              void* dtv, void* workspace, size_t workspace_bytes, int B, int H, int Lq, int Lk, int D,
              const int64_t* strides, float scale, int dtype, void* stream) {
+    return sjvp_bwd_parts(SJVP_BWD_ALL, q, k, v, tq, tk, tv, o, to, dO, dTO, lse, mu, dq, dk, dv, dtq, dtk,
+                          dtv, workspace, workspace_bytes, B, H, Lq, Lk, D, strides, scale, dtype, stream);
+}
+
+int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const void* tq,
+                   const void* tk, const void* tv, const void* o, const void* to, const void* dO,
+                   const void* dTO, const float* lse, const float* mu, void* dq, void* dk, void* dv,
+                   void* dtq, void* dtk, void* dtv, void* workspace, size_t workspace_bytes, int B,
+                   int H, int Lq, int Lk, int D, const int64_t* strides, float scale, int dtype,
+                   void* stream) {
+    if (parts < SJVP_BWD_ROW || parts > SJVP_BWD_ALL) return SJVP_ERR_PARTS;
     if (!dO && !dTO) return SJVP_ERR_COTANGENT;
     const bool has_do = dO != nullptr, has_g = dTO != nullptr;
     if (!q || !k || !v || !o || !lse || !dq || !dk || !dv || !strides) return SJVP_ERR_NULL;
@@ -238,8 +251,8 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, s)
-                              : bwd_dtype<Fp16>(p, B * H, has_do, has_g, s);
+    return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, parts, s)
+                              : bwd_dtype<Fp16>(p, B * H, has_do, has_g, parts, s);
 }
 
 const char* sjvp_strerror(int status) {
@@ -252,6 +265,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than sjvp_bwd_workspace_bytes()";
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
+        case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
         default: return "unknown sjvp status";
     }
 }

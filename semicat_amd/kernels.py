@@ -132,11 +132,14 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
 
 
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
-                           scale: Optional[float] = None, grads=None):
+                           scale: Optional[float] = None, grads=None, workspace=None,
+                           parts: int = _lib.SJVP_BWD_ALL):
     """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
     Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
     tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
-    (the tangent three may be None without dTO)."""
+    (the tangent three may be None without dTO); ``workspace`` a uint8 device buffer of at least
+    ``sjvp_bwd_workspace_bytes`` bytes (allocated here otherwise).  ``parts`` selects the launches
+    (profiling only: SJVP_BWD_COL alone needs the workspace an earlier SJVP_BWD_ROW call filled)."""
     dtype_tag = _require_gpu(q)
     if dO is None and dTO is None:
         raise ValueError("attention_jvp_backward needs a cotangent on o, on to, or on both")
@@ -189,11 +192,14 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         dtq = dtk = dtv = None
     lib = _lib.load()
     nbytes = lib.sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype_tag)
-    workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
+    if workspace is None:
+        workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
+    elif workspace.dtype != torch.uint8 or workspace.numel() < nbytes or workspace.device != dev:
+        raise AssertionError(f"workspace must be a uint8 tensor of >= {nbytes} bytes on {dev}")
     tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.sjvp_bwd(*(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
+        rc = lib.sjvp_bwd_parts(int(parts), *(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
                           *(_ptr(t) for t in tensors[10:]), _ptr(workspace), nbytes, B, H, Lq, Lk, D,
                           _strides(tensors), float(scale) if scale else 0.0, dtype_tag,
                           ctypes.c_void_p(stream))

@@ -145,7 +145,7 @@ def test_library_exports_every_declared_symbol(repo_root):
     assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
     assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4
     assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4
-    for code in range(0, -8, -1):
+    for code in range(0, -9, -1):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
