@@ -30,7 +30,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
-# kernel of --calib-copy).  Commands and raw figures: profiles/.
+# kernel of --calib-copy).
 MEASURED_TRAFFIC_BYTES = {
     "fwd_kernel": (2 * 37004.0 + 25344.0) * 1024,      # FETCH_SIZE counts 2 KiB per unit on the copy
     "bwd_row_kernel": (2 * 61983.0 + 25728.0) * 1024,  # kernel (131089 for 262144 KiB), WRITE_SIZE 1 KiB
@@ -205,7 +205,7 @@ def main() -> int:
         roofline = {"bound": "mfma", "achieved": dk["TFLOPs"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": dk["TFLOPs"] / PEAK_BF16_TFLOPS}
     # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-    # this script (scaled by the same counters on the --calib-copy kernel); see profiles/.
+    # this script (scaled by the same counters on the --calib-copy kernel).
     roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom)
     roofline["kernel"] = dom
     roofline["ms"] = dk["ms"]
