@@ -58,10 +58,14 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
 // the workgroup's own rows (160 KB per CU; the forward keeps two workgroups per CU resident).
 template <int HD>
 struct Ring {
+#ifdef SJVP_X_RINGS
+    static constexpr int fwd = 3, fwd_primal = 4, row = 2, col = 2;
+#else
     static constexpr int fwd = HD == 128 ? 2 : 4;         // with tangents (four slabs per stage)
     static constexpr int fwd_primal = 4;                  // primal only (two slabs per stage)
     static constexpr int row = 3;
     static constexpr int col = HD == 128 ? 3 : 4;
+#endif
 };
 
 template <typename T, int HD, bool DMA>
@@ -166,7 +170,7 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.Lk = Lk;
     p.D = D;
     p.Lr = round_up(Lq, 128);
-    p.q_blocks = p.Lr / 128;
+    p.q_blocks = p.Lr / kOwned;  // covers every statistic row below Lr
     p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
@@ -242,8 +246,8 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
     p.Lk = Lk;
     p.D = D;
     p.Lr = round_up(Lq, 128);
-    p.q_blocks = p.Lr / 128;
-    p.k_blocks = round_up(Lk, 128) / 128;
+    p.q_blocks = p.Lr / kOwned;
+    p.k_blocks = round_up(Lk, kOwned) / kOwned;
     p.lse2 = static_cast<float*>(workspace);
     p.s4 = p.lse2 + (size_t)B * H * p.Lr;
     p.s7d = p.s4 + (size_t)B * H * p.Lr;

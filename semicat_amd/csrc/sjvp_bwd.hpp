@@ -34,7 +34,7 @@ struct BwdParams {
     float* s4;    // workspace [B*H][Lr]  rowsum(G*O)
     float* s7d;   // workspace [B*H][Lr]  rowsum(G*TO) + rowsum(dO*O)
     int H, Lq, Lk, D, Lr;
-    int q_blocks, k_blocks;  // ceil(L / 128)
+    int q_blocks, k_blocks;  // workgroups per (batch, head) along the owned axis
     float scale;
     int vec;
 };
@@ -42,8 +42,8 @@ struct BwdParams {
 // ---------------------------------------------------------------------------------------------
 // Row-owned kernel: dQ (and dQ_dot).  Tiles are transposed (rows = keys in registers, columns =
 // this wave's queries in lanes), so the row statistics are per-lane scalars.
-// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's 128 rows of Q, O (, Q_dot, G, TO)
-// (, dO), 4 slabs each][lse and mu of those rows][ring of K, V (, K_dot, V_dot) stages]; the ring
+// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's rows of Q, O (, Q_dot, G, TO)
+// (, dO), one slab per wave each][lse and mu of those rows][ring of K, V (, K_dot, V_dot) stages]; the ring
 // doubles as store staging after the last stage.
 template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
 struct RowSmem {
@@ -51,7 +51,7 @@ struct RowSmem {
     static constexpr int nt = HAS_G ? 4 : 2;
     static constexpr int slot = nt * Slab<HD>::elems;
     static constexpr int n_own = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
-    static constexpr int own = own_lds ? n_own * 4 * Slab<HD>::elems : 0;
+    static constexpr int own = own_lds ? n_own * kWaves * Slab<HD>::elems : 0;
     static constexpr int stat = own_lds ? 2 * kOwned * 2 : 0;  // two float arrays, in elem_t units
     static constexpr int bytes = (own + stat + R * slot) * (int)sizeof(elem_t);
 };
@@ -65,9 +65,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     float* own_stat = reinterpret_cast<float*>(own + SM::own);
     elem_t* ring = own + SM::own + SM::stat;
     // own tensor order: Q, O, [Q_dot, G, TO], [dO]
-    constexpr int oQ = 0, oO = 4 * Slab<HD>::elems, oTQ = 8 * Slab<HD>::elems,
-                  oG = 12 * Slab<HD>::elems, oTO = 16 * Slab<HD>::elems,
-                  oDO = (HAS_G ? 20 : 8) * Slab<HD>::elems;
+    constexpr int oQ = 0, oO = kWaves * Slab<HD>::elems, oTQ = 2 * kWaves * Slab<HD>::elems,
+                  oG = 3 * kWaves * Slab<HD>::elems, oTO = 4 * kWaves * Slab<HD>::elems,
+                  oDO = (HAS_G ? 5 : 2) * kWaves * Slab<HD>::elems;
 
     constexpr int KC = HD / 16;
     constexpr int DT = HD / 32;
@@ -81,6 +81,8 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     const int qb = blockIdx.x % p.q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
+    SlabLane<HD> ln;
+    ln.init(tid);
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -94,9 +96,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         const int r0 = qb * kOwned;
         auto own_fill = [&](int off, const TensorView& t) {
 #pragma unroll
-            for (int s4 = 0; s4 < 4; ++s4)
-                fill_slab<HD, true>(own + off + s4 * Slab<HD>::elems, t.head(b, h), t.sl, r0 + 32 * s4,
-                                    p.Lq, p.D, true, tid);
+            for (int s4 = 0; s4 < kWaves; ++s4)
+                fill_slab<HD, true>(ln, own + off + s4 * Slab<HD>::elems, t.head(b, h), t.sl, r0 + 32 * s4,
+                                    p.Lq, p.D, true);
         };
         own_fill(oQ, p.q);
         own_fill(oO, p.o);
@@ -137,7 +139,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
         mu = (qvalid && HAS_G) ? p.mu[so] : 0.f;
         if constexpr (DMA) {
-            // retire these loads before the first LDS-DMA copy so that wait_vmcnt() only has the
+            // retire these loads before the first LDS-DMA copy so that wait_stages() only has the
             // ring's traffic to count
             asm volatile("" : "+v"(lse2), "+v"(mu));
 #pragma unroll
@@ -187,11 +189,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     auto issue = [&](int stage) {
         elem_t* slot = ring + (stage % R) * SM::slot;
         const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(slot, kg, p.k.sl, row0, p.Lk, p.D, vec, tid);
-        fill_slab<HD, DMA>(slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec, tid);
+        fill_slab<HD, DMA>(ln, slot, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, DMA>(ln, slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD, DMA>(slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec, tid);
-            fill_slab<HD, DMA>(slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec, tid);
+            fill_slab<HD, DMA>(ln, slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, DMA>(ln, slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -264,7 +266,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         int issued = 0;
         for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
         if constexpr (OWN_LDS) {
-            wait_vmcnt(issued * SPT);  // the own rows were issued before these stages
+            wait_stages<SPT>(issued);  // the own rows were issued before these stages
             __syncthreads();
             const int sw = wave * Slab<HD>::elems;
             read_b_operands<HD>(qB, own + oQ + sw, x, hf);
@@ -288,7 +290,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     }
     for (int i = 0; i < n; ++i) {
         if constexpr (DMA) {
-            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
+            wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
             __syncthreads();
             if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
         } else {
@@ -332,8 +334,8 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
 // Column-owned kernel: a wavefront owns 32 keys and streams the queries.  DO_K selects dK (and
 // dK_dot), DO_V selects dV (and dV_dot); DT0/NDT select the 32-wide head-dimension tiles that are
 // accumulated (at HD = 128 the work is split to stay inside the register file).
-// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's 128 rows of K, V (, K_dot, V_dot),
-// 4 slabs each][ring of Q (, Q_dot, G) (, dO) stages, each followed by its row statistics]; the
+// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's rows of K, V (, K_dot, V_dot),
+// one slab per wave each][ring of Q (, Q_dot, G) (, dO) stages, each followed by its row statistics]; the
 // ring doubles as store staging after the last stage.
 template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
 struct ColSmem {
@@ -341,7 +343,7 @@ struct ColSmem {
     static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
     static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
     static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
-    static constexpr int own = own_lds ? (HAS_G ? 4 : 2) * 4 * Slab<HD>::elems : 0;
+    static constexpr int own = own_lds ? (HAS_G ? 4 : 2) * kWaves * Slab<HD>::elems : 0;
     static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
 };
 
@@ -370,9 +372,16 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     const int kb = blockIdx.x % p.k_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
-    // LDS-DMA instructions per stage issued by this wave: the tensors, plus one 4-byte copy of two
-    // statistic arrays by waves 0 and 1
-    const int spt = SM::nt * Slab<HD>::per_thread + (wave < 2 ? 1 : 0);
+    SlabLane<HD> ln;
+    ln.init(tid);
+    // LDS-DMA instructions per stage issued by every wave: the tensors plus one 4-byte copy of
+    // statistics
+    constexpr int SPT = SM::nt * Slab<HD>::per_thread + 1;
+#ifdef SJVP_X_STAGGER
+    if ((blockIdx.x / 8) & 1) {
+        for (int i_ = 0; i_ < SJVP_X_STAGGER; ++i_) __builtin_amdgcn_s_sleep(64);
+    }
+#endif
     const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;
@@ -382,9 +391,9 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
         const int r0 = kb * kOwned;
         auto own_fill = [&](int idx, const TensorView& t) {
 #pragma unroll
-            for (int s4 = 0; s4 < 4; ++s4)
-                fill_slab<HD, true>(own + (4 * idx + s4) * Slab<HD>::elems, t.head(b, h), t.sl,
-                                    r0 + 32 * s4, p.Lk, p.D, true, tid);
+            for (int s4 = 0; s4 < kWaves; ++s4)
+                fill_slab<HD, true>(ln, own + (kWaves * idx + s4) * Slab<HD>::elems, t.head(b, h), t.sl,
+                                    r0 + 32 * s4, p.Lk, p.D, true);
         };
         own_fill(0, p.k);
         own_fill(1, p.v);
@@ -430,23 +439,27 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     auto issue = [&](int stage) {
         elem_t* slot = ring + (stage % R) * SM::slot;
         const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(slot, qg, p.q.sl, row0, p.Lq, p.D, vec, tid);
+        fill_slab<HD, DMA>(ln, slot, qg, p.q.sl, row0, p.Lq, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD, DMA>(slot + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec, tid);
-            fill_slab<HD, DMA>(slot + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec, tid);
+            fill_slab<HD, DMA>(ln, slot + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec);
+            fill_slab<HD, DMA>(ln, slot + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec);
         }
-        if constexpr (HAS_DO) fill_slab<HD, DMA>(slot + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec, tid);
+        if constexpr (HAS_DO) fill_slab<HD, DMA>(ln, slot + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec);
         // Row statistics of the stage (rows < Lr are defined in all four arrays; rows beyond Lq
         // hold finite values and multiply zero rows of Q, Q_dot, G, dO below).
         float* st = reinterpret_cast<float*>(slot + oST);
         const int64_t so = (int64_t)bh * p.Lr + row0 + (lane & 31);
-        if (wave < 2) {
-            const float* src = wave == 0 ? (hf == 0 ? p.lse2 : p.mu) : (hf == 0 ? p.s4 : p.s7d);
+        // the four arrays (lse2, mu, s4, s7d) are dealt to the waves, 32 lanes each; every wave
+        // issues exactly one 4-byte LDS-DMA instruction
+        constexpr int APW = 4 / kWaves;  // arrays per wave
+        const int arr = wave * APW + hf;
+        if (hf < APW) {
+            const float* src = arr == 0 ? p.lse2 : arr == 1 ? p.mu : arr == 2 ? p.s4 : p.s7d;
+            if (arr == 1 && !HAS_G) src = p.s4;  // mu is not used without the tangent cotangent
             if constexpr (DMA) {
-                const uint32_t base = lds_addr(st) + (uint32_t)(wave * 64 * 4);
-                if (HAS_G || !(wave == 0 && hf == 1)) dma4(src + so, base);
+                dma4(src + so, lds_addr(st) + (uint32_t)(wave * APW * 32 * 4));
             } else {
-                st[wave * 64 + lane] = (HAS_G || !(wave == 0 && hf == 1)) ? src[so] : 0.f;
+                st[arr * 32 + (lane & 31)] = src[so];
             }
         }
     };
@@ -556,19 +569,20 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
         int issued = 0;
         for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
         if constexpr (OWN_LDS) {
-            wait_vmcnt(issued * spt);  // the own rows were issued before these stages
+            wait_stages<SPT>(issued);  // the own rows were issued before these stages
             __syncthreads();
             read_b_operands<HD>(kB, own + wave * Slab<HD>::elems, x, hf);
-            if constexpr (DO_K) read_b_operands<HD>(vB, own + (4 + wave) * Slab<HD>::elems, x, hf);
+            if constexpr (DO_K) read_b_operands<HD>(vB, own + (kWaves + wave) * Slab<HD>::elems, x, hf);
             if constexpr (HAS_G) {
-                read_b_operands<HD>(tkB, own + (8 + wave) * Slab<HD>::elems, x, hf);
-                if constexpr (DO_K) read_b_operands<HD>(tvB, own + (12 + wave) * Slab<HD>::elems, x, hf);
+                read_b_operands<HD>(tkB, own + (2 * kWaves + wave) * Slab<HD>::elems, x, hf);
+                if constexpr (DO_K)
+                    read_b_operands<HD>(tvB, own + (3 * kWaves + wave) * Slab<HD>::elems, x, hf);
             }
         }
     }
     for (int i = 0; i < n; ++i) {
         if constexpr (DMA) {
-            wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * spt);
+            wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
             __syncthreads();
             if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
         } else {

@@ -42,8 +42,11 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef uint16_t elem_t;  // storage type of one 16-bit element, whatever its format
 
-constexpr int kThreads = 256;  // 4 wavefronts per workgroup
-constexpr int kWaves = 4;
+#ifndef SJVP_WAVES
+#define SJVP_WAVES 4
+#endif
+constexpr int kWaves = SJVP_WAVES;  // wavefronts per workgroup (2 or 4)
+constexpr int kThreads = 64 * kWaves;
 constexpr int kOwned = 32 * kWaves;  // positions of the owned axis per workgroup
 constexpr int kStageRows = 32;       // rows of the looped axis per stage
 constexpr float kLog2e = 1.4426950408889634f;
@@ -166,52 +169,74 @@ __device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_base) {
                  : "memory");
 }
 
-// s_waitcnt vmcnt(n) for a run-time n (clamped to the encodable 0..63): at most n of this wave's
-// vector-memory operations may still be outstanding afterwards.  Loads and LDS-DMA copies retire
-// in issue order, so this guarantees that all but the n most recent ones have landed.
-__device__ __forceinline__ void wait_vmcnt(int n) {
-#define SJVP_VM(k) \
-    case k: __builtin_amdgcn_s_waitcnt(((k) & 15) | (((k) >> 4) << 14) | 0x0F70); break;
-    switch (n) {
-        SJVP_VM(0) SJVP_VM(1) SJVP_VM(2) SJVP_VM(3) SJVP_VM(4) SJVP_VM(5) SJVP_VM(6) SJVP_VM(7)
-        SJVP_VM(8) SJVP_VM(9) SJVP_VM(10) SJVP_VM(11) SJVP_VM(12) SJVP_VM(13) SJVP_VM(14)
-        SJVP_VM(15) SJVP_VM(16) SJVP_VM(17) SJVP_VM(18) SJVP_VM(19) SJVP_VM(20) SJVP_VM(21)
-        SJVP_VM(22) SJVP_VM(23) SJVP_VM(24) SJVP_VM(25) SJVP_VM(26) SJVP_VM(27) SJVP_VM(28)
-        SJVP_VM(29) SJVP_VM(30) SJVP_VM(31) SJVP_VM(32) SJVP_VM(33) SJVP_VM(34) SJVP_VM(35)
-        SJVP_VM(36) SJVP_VM(37) SJVP_VM(38) SJVP_VM(39) SJVP_VM(40) SJVP_VM(41) SJVP_VM(42)
-        SJVP_VM(43) SJVP_VM(44) SJVP_VM(45) SJVP_VM(46) SJVP_VM(47) SJVP_VM(48)
-        default: __builtin_amdgcn_s_waitcnt(0x0F70 | 15 | (3 << 14)); break;  // vmcnt(63)
+// s_waitcnt vmcnt(ahead * SPT): at most `ahead` later stages (SPT vector-memory instructions each,
+// SPT a compile-time constant) of this wave's copies may still be outstanding afterwards.  Loads and
+// LDS-DMA copies retire in issue order, so everything issued before those stages has landed.
+// `ahead` is wave-uniform and small (at most the ring depth); counts beyond the 6-bit field are
+// clamped, which only makes the wait stricter.
+template <int SPT>
+__device__ __forceinline__ void wait_stages(int ahead) {
+#define SJVP_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) > 63 ? 63 : (n)) & 15) | ((((n) > 63 ? 63 : (n)) >> 4) << 14) | 0x0F70)
+    switch (ahead) {
+        case 0: SJVP_VMCNT(0); break;
+        case 1: SJVP_VMCNT(SPT); break;
+        case 2: SJVP_VMCNT(2 * SPT); break;
+        case 3: SJVP_VMCNT(3 * SPT); break;
+        case 4: SJVP_VMCNT(4 * SPT); break;
+        case 5: SJVP_VMCNT(5 * SPT); break;
+        case 6: SJVP_VMCNT(6 * SPT); break;
+        default: SJVP_VMCNT(7 * SPT); break;
     }
-#undef SJVP_VM
+#undef SJVP_VMCNT
 }
+
+// Per-thread geometry of a slab copy: which 16-byte chunk positions of a slab this thread fills and
+// which (row, column) of the source they hold.  Computed once per kernel.
+template <int HD>
+struct SlabLane {
+    static constexpr int N = Slab<HD>::per_thread;
+    int r[N];        // slab row
+    int c8[N];       // source column (elements) of the chunk
+    int pos8[N];     // element offset of the chunk position inside the slab
+    uint32_t wbase[N];  // byte offset, inside the slab, of the wave's first chunk position
+    bool on[N];      // the position exists (slabs smaller than the workgroup)
+    __device__ __forceinline__ void init(int tid) {
+        constexpr int CH = HD / 8;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int pos = tid + i * kThreads;
+            r[i] = pos / CH;
+            c8[i] = 8 * ((pos % CH) ^ swz<HD>(r[i]));
+            pos8[i] = pos * 8;
+            wbase[i] = (uint32_t)((pos & ~63) * 16);
+            on[i] = pos < Slab<HD>::chunks;
+        }
+    }
+};
 
 // Copy stage rows row0 .. row0+31 of one [L][D] head slice into a slab (swizzled), zero-filled
 // beyond L and beyond D.  DMA = true: asynchronous LDS-DMA (needs `vec` inputs); the caller retires
-// it with wait_vmcnt + barrier; exactly Slab<HD>::per_thread LDS-DMA instructions are issued by
-// every wave when HD >= 64.  DMA = false: synchronous copy through registers (any alignment).
+// it with wait_stages + barrier; exactly Slab<HD>::per_thread LDS-DMA instructions are issued by
+// every wave when the slab has at least one chunk per thread.  DMA = false: synchronous copy through
+// registers (any alignment).
 template <int HD, bool DMA>
-__device__ __forceinline__ void fill_slab(elem_t* slab, const elem_t* g, int64_t sl, int row0, int L,
-                                          int D, bool vec, int tid) {
-    constexpr int CH = HD / 8;
+__device__ __forceinline__ void fill_slab(const SlabLane<HD>& ln, elem_t* slab, const elem_t* g,
+                                          int64_t sl, int row0, int L, int D, bool vec) {
 #pragma unroll
-    for (int i = 0; i < Slab<HD>::per_thread; ++i) {
-        const int pos = tid + i * kThreads;  // chunk position inside the slab
-        if (Slab<HD>::chunks % kThreads != 0 && pos >= Slab<HD>::chunks) break;
-        const int r = pos / CH;
-        const int c = (pos % CH) ^ swz<HD>(r);
-        const int row = row0 + r;
-        const bool valid = (row < L) && (8 * c < D);
+    for (int i = 0; i < SlabLane<HD>::N; ++i) {
+        if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) break;
+        const int row = row0 + ln.r[i];
+        const bool valid = (row < L) && (ln.c8[i] < D);
         if constexpr (DMA) {
-            // every lane of the wave writes base + 16*lane: base is the slab address of the wave's
-            // first chunk position
-            const uint32_t base = lds_addr(slab) + (uint32_t)((pos & ~63) * 16);
+            // every lane of the wave writes base + 16*lane
             if (valid) {
-                dma16(g + (int64_t)row * sl + 8 * c, base);
+                dma16(g + (int64_t)row * sl + ln.c8[i], lds_addr(slab) + ln.wbase[i]);
             } else {
-                *reinterpret_cast<u32x4*>(slab + pos * 8) = u32x4{0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) = u32x4{0u, 0u, 0u, 0u};
             }
         } else {
-            *reinterpret_cast<u32x4*>(slab + pos * 8) = load8(g + (int64_t)row * sl, 8 * c, D, row < L, vec);
+            *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) =
+                load8(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
         }
     }
 }

@@ -22,19 +22,19 @@ struct FwdParams {
     float* mu;
     float* li;
     int H, Lq, Lk, D, Lr;
-    int q_blocks;  // ceil(Lq / 128)
+    int q_blocks;  // workgroups per (batch, head): Lr / (32 * waves per workgroup)
     float scale;
     int vec;  // all tensors 16-byte aligned, strides % 8 == 0, D % 8 == 0
 };
 
-// LDS layout: [own: Q (and Q_dot) rows of the workgroup, 4 slabs each - LDS-DMA path only]
+// LDS layout: [own: Q (and Q_dot) rows of the workgroup, one slab per wave - LDS-DMA path only]
 //             [ring: R slots of K, V (, K_dot, V_dot) stage slabs]
 // After the last stage the ring memory doubles as the per-wave staging tiles of the output stores.
 template <int HD, int R, bool JVP, bool DMA>
 struct FwdSmem {
     static constexpr int nt = JVP ? 4 : 2;                      // tensors per stage
     static constexpr int slot = nt * Slab<HD>::elems;            // elements per ring slot
-    static constexpr int own = DMA ? (JVP ? 2 : 1) * 4 * Slab<HD>::elems : 0;
+    static constexpr int own = DMA ? (JVP ? 2 : 1) * kWaves * Slab<HD>::elems : 0;
     static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
     static_assert(!DMA || R * slot >= kWaves * StoreStage<HD>::elems, "ring too small to stage stores");
 };
@@ -66,6 +66,8 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     const int qb = blockIdx.x % p.q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
+    SlabLane<HD> ln;
+    ln.init(tid);
     const int qrow = qb * kOwned + wave * 32 + x;  // the query this lane owns
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -77,12 +79,12 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     if constexpr (DMA) {
         const int r0 = qb * kOwned;
 #pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-            fill_slab<HD, true>(own + s4 * Slab<HD>::elems, p.q.head(b, h), p.q.sl, r0 + 32 * s4, p.Lq,
-                                p.D, true, tid);
+        for (int s4 = 0; s4 < kWaves; ++s4) {
+            fill_slab<HD, true>(ln, own + s4 * Slab<HD>::elems, p.q.head(b, h), p.q.sl, r0 + 32 * s4, p.Lq,
+                                p.D, true);
             if constexpr (JVP)
-                fill_slab<HD, true>(own + (4 + s4) * Slab<HD>::elems, p.tq.head(b, h), p.tq.sl,
-                                    r0 + 32 * s4, p.Lq, p.D, true, tid);
+                fill_slab<HD, true>(ln, own + (kWaves + s4) * Slab<HD>::elems, p.tq.head(b, h), p.tq.sl,
+                                    r0 + 32 * s4, p.Lq, p.D, true);
         }
     } else {
         const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
@@ -102,11 +104,11 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     auto issue = [&](int stage) {
         elem_t* slot = ring + (stage % R) * SM::slot;
         const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(slot, kg, p.k.sl, row0, p.Lk, p.D, vec, tid);
-        fill_slab<HD, DMA>(slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec, tid);
+        fill_slab<HD, DMA>(ln, slot, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, DMA>(ln, slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (JVP) {
-            fill_slab<HD, DMA>(slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec, tid);
-            fill_slab<HD, DMA>(slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec, tid);
+            fill_slab<HD, DMA>(ln, slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, DMA>(ln, slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -225,10 +227,10 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
         for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
         // the owned rows were issued before these stages: they have landed once at most the
         // stages' copies are outstanding
-        wait_vmcnt(issued * SPT);
+        wait_stages<SPT>(issued);
         __syncthreads();
         read_b_operands<HD>(qB, own + wave * Slab<HD>::elems, x, hf);
-        if constexpr (JVP) read_b_operands<HD>(tqB, own + (4 + wave) * Slab<HD>::elems, x, hf);
+        if constexpr (JVP) read_b_operands<HD>(tqB, own + (kWaves + wave) * Slab<HD>::elems, x, hf);
     }
     using one_t = std::integral_constant<int, 1>;
     using two_t = std::integral_constant<int, 2>;
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
         for (int i = 0, last = 0; i < n; i = last + 1) {
             // pair up with stage i+1 only if it has been issued already
             last = (i + 1 < next) ? i + 1 : i;
-            wait_vmcnt((next - 1 - last) * SPT);
+            wait_stages<SPT>(next - 1 - last);
             __syncthreads();  // stages i..last have landed for every wave; stages < i are consumed
             while (next < n && next < i + R) issue(next++);
             if (!wave_active) continue;
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     } else {
         for (int i = 0; i < n; ++i) {
             if constexpr (DMA) {
-                wait_vmcnt((ring_issued_before(i, R, n) - 1 - i) * SPT);
+                wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
                 __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
                 if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
             } else {
