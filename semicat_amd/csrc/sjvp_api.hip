@@ -6,7 +6,9 @@
 #include <math.h>
 
 #include "sjvp_bwd.hpp"
+#include "sjvp_bwd_fused.hpp"
 #include "sjvp_fwd.hpp"
+#include "sjvp_fwd16.hpp"
 
 using namespace sjvp;
 
@@ -41,7 +43,8 @@ int check_common(int B, int H, int Lq, int Lk, int D, int dtype) {
 }
 
 template <typename K>
-int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params) {
+int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params,
+           int threads = kThreads) {
     if (smem_bytes > 64 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -50,7 +53,7 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
             return SJVP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem_bytes, stream, params);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem_bytes, stream, params);
     return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
 }
 
@@ -58,14 +61,11 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
 // the workgroup's own rows (160 KB per CU; the forward keeps two workgroups per CU resident).
 template <int HD>
 struct Ring {
-#ifdef SJVP_X_RINGS
-    static constexpr int fwd = 3, fwd_primal = 4, row = 2, col = 2;
-#else
     static constexpr int fwd = HD == 128 ? 2 : 4;         // with tangents (four slabs per stage)
     static constexpr int fwd_primal = 4;                  // primal only (two slabs per stage)
     static constexpr int row = 3;
     static constexpr int col = HD == 128 ? 3 : 4;
-#endif
+    static constexpr int fused = 3;
 };
 
 template <typename T, int HD, bool DMA>
@@ -77,10 +77,33 @@ int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     return launch(fwd_kernel<T, HD, RP, false, DMA>, grid, FwdSmem<HD, RP, false, DMA>::bytes, stream, p);
 }
 
+#ifndef SJVP_F16_R
+#define SJVP_F16_R 2
+#endif
+#ifndef SJVP_F16_OCC
+#define SJVP_F16_OCC 2
+#endif
+template <typename T, int HD>
+int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
+    constexpr int R = HD == 128 ? 2 : SJVP_F16_R;
+    constexpr int RP = 4;
+    constexpr int OCC = HD == 128 ? 2 : SJVP_F16_OCC;
+    if (jvp)
+        return launch(fwd16_kernel<T, HD, R, true, OCC>, grid, Fwd16Smem<HD, R, true>::bytes, stream, p,
+                      kThreads16);
+    return launch(fwd16_kernel<T, HD, RP, false, OCC>, grid, Fwd16Smem<HD, RP, false>::bytes, stream, p,
+                  kThreads16);
+}
+
 template <typename T>
 int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
     if (p.vec) {
+#ifndef SJVP_NO_F16
+        if (p.D <= 32) return fwd16_hd<T, 32>(p, grid, jvp, stream);
+        if (p.D <= 64) return fwd16_hd<T, 64>(p, grid, jvp, stream);
+        return fwd16_hd<T, 128>(p, grid, jvp, stream);
+#endif
         if (p.D <= 32) return fwd_hd<T, 32, true>(p, grid, jvp, stream);
         if (p.D <= 64) return fwd_hd<T, 64, true>(p, grid, jvp, stream);
         return fwd_hd<T, 128, true>(p, grid, jvp, stream);
@@ -94,6 +117,14 @@ template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
 int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     constexpr int R = DMA ? Ring<HD>::row : 1;
     constexpr int CR = DMA ? Ring<HD>::col : 1;
+    if constexpr (DMA && HD <= 64) {
+        // short key axis: one launch, one workgroup per (batch, head)
+        if (parts == SJVP_BWD_ALL && p.Lk <= kOwned) {
+            constexpr int FR = Ring<HD>::fused;
+            return launch(bwd_fused_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
+                          FusedSmem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p);
+        }
+    }
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.
     int rc = SJVP_OK;
     if (parts & SJVP_BWD_ROW)

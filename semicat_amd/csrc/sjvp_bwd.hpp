@@ -53,7 +53,8 @@ struct RowSmem {
     static constexpr int n_own = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
     static constexpr int own = own_lds ? n_own * kWaves * Slab<HD>::elems : 0;
     static constexpr int stat = own_lds ? 2 * kOwned * 2 : 0;  // two float arrays, in elem_t units
-    static constexpr int bytes = (own + stat + R * slot) * (int)sizeof(elem_t);
+    static constexpr int sink = (own + stat + R * slot) * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSinkBytes;
 };
 
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid);
+    ln.init(tid, smem_raw + SM::sink);
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -344,7 +345,8 @@ struct ColSmem {
     static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
     static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
     static constexpr int own = own_lds ? (HAS_G ? 4 : 2) * kWaves * Slab<HD>::elems : 0;
-    static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
+    static constexpr int sink = (own + R * slot) * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSinkBytes;
 };
 
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT,
@@ -373,15 +375,10 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid);
+    ln.init(tid, smem_raw + SM::sink);
     // LDS-DMA instructions per stage issued by every wave: the tensors plus one 4-byte copy of
     // statistics
     constexpr int SPT = SM::nt * Slab<HD>::per_thread + 1;
-#ifdef SJVP_X_STAGGER
-    if ((blockIdx.x / 8) & 1) {
-        for (int i_ = 0; i_ < SJVP_X_STAGGER; ++i_) __builtin_amdgcn_s_sleep(64);
-    }
-#endif
     const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;

@@ -57,6 +57,10 @@ struct Bf16 {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                      __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
         bf16x2 v = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, v);
@@ -69,6 +73,10 @@ struct Bf16 {
 struct Fp16 {
     static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                     __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -169,26 +177,30 @@ __device__ __forceinline__ void dma4(const void* gptr, uint32_t lds_base) {
                  : "memory");
 }
 
-// s_waitcnt vmcnt(ahead * SPT): at most `ahead` later stages (SPT vector-memory instructions each,
+// s_waitcnt vmcnt(ahead * SPT + EXTRA): at most `ahead` later stages (SPT vector-memory instructions each,
 // SPT a compile-time constant) of this wave's copies may still be outstanding afterwards.  Loads and
 // LDS-DMA copies retire in issue order, so everything issued before those stages has landed.
+// EXTRA counts other vector-memory instructions (stores) known to have been issued after them.
 // `ahead` is wave-uniform and small (at most the ring depth); counts beyond the 6-bit field are
 // clamped, which only makes the wait stricter.
-template <int SPT>
+template <int SPT, int EXTRA = 0>
 __device__ __forceinline__ void wait_stages(int ahead) {
 #define SJVP_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) > 63 ? 63 : (n)) & 15) | ((((n) > 63 ? 63 : (n)) >> 4) << 14) | 0x0F70)
     switch (ahead) {
-        case 0: SJVP_VMCNT(0); break;
-        case 1: SJVP_VMCNT(SPT); break;
-        case 2: SJVP_VMCNT(2 * SPT); break;
-        case 3: SJVP_VMCNT(3 * SPT); break;
-        case 4: SJVP_VMCNT(4 * SPT); break;
-        case 5: SJVP_VMCNT(5 * SPT); break;
-        case 6: SJVP_VMCNT(6 * SPT); break;
-        default: SJVP_VMCNT(7 * SPT); break;
+        case 0: SJVP_VMCNT(EXTRA); break;
+        case 1: SJVP_VMCNT(SPT + EXTRA); break;
+        case 2: SJVP_VMCNT(2 * SPT + EXTRA); break;
+        case 3: SJVP_VMCNT(3 * SPT + EXTRA); break;
+        case 4: SJVP_VMCNT(4 * SPT + EXTRA); break;
+        case 5: SJVP_VMCNT(5 * SPT + EXTRA); break;
+        case 6: SJVP_VMCNT(6 * SPT + EXTRA); break;
+        default: SJVP_VMCNT(7 * SPT + EXTRA); break;
     }
 #undef SJVP_VMCNT
 }
+
+// Every shared-memory layout ends with this many bytes that LDS-DMA placeholders may overwrite.
+constexpr int kSinkBytes = 256;
 
 // Per-thread geometry of a slab copy: which 16-byte chunk positions of a slab this thread fills and
 // which (row, column) of the source they hold.  Computed once per kernel.
@@ -200,7 +212,9 @@ struct SlabLane {
     int pos8[N];     // element offset of the chunk position inside the slab
     uint32_t wbase[N];  // byte offset, inside the slab, of the wave's first chunk position
     bool on[N];      // the position exists (slabs smaller than the workgroup)
-    __device__ __forceinline__ void init(int tid) {
+    uint32_t sink;   // LDS byte address of kSinkBytes that nothing reads
+    __device__ __forceinline__ void init(int tid, const void* sink_lds) {
+        sink = lds_addr(sink_lds);
         constexpr int CH = HD / 8;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
@@ -217,14 +231,20 @@ struct SlabLane {
 // Copy stage rows row0 .. row0+31 of one [L][D] head slice into a slab (swizzled), zero-filled
 // beyond L and beyond D.  DMA = true: asynchronous LDS-DMA (needs `vec` inputs); the caller retires
 // it with wait_stages + barrier; exactly Slab<HD>::per_thread LDS-DMA instructions are issued by
-// every wave when the slab has at least one chunk per thread.  DMA = false: synchronous copy through
-// registers (any alignment).
+// every wave: a wave none of whose lanes has a row below L, or whose threads lie beyond a slab
+// smaller than the workgroup, issues a 4-byte placeholder copy into the sink instead, so that the
+// vmcnt arithmetic of wait_stages stays exact.  DMA = false: synchronous copy through registers
+// (any alignment).
 template <int HD, bool DMA>
 __device__ __forceinline__ void fill_slab(const SlabLane<HD>& ln, elem_t* slab, const elem_t* g,
                                           int64_t sl, int row0, int L, int D, bool vec) {
+    const bool ragged = row0 + kStageRows > L;  // uniform
 #pragma unroll
     for (int i = 0; i < SlabLane<HD>::N; ++i) {
-        if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) break;
+        if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) {  // wave-uniform: a wave beyond the slab
+            if constexpr (DMA) dma4(g, ln.sink);
+            break;
+        }
         const int row = row0 + ln.r[i];
         const bool valid = (row < L) && (ln.c8[i] < D);
         if constexpr (DMA) {
@@ -234,6 +254,7 @@ __device__ __forceinline__ void fill_slab(const SlabLane<HD>& ln, elem_t* slab, 
             } else {
                 *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) = u32x4{0u, 0u, 0u, 0u};
             }
+            if (ragged && __builtin_amdgcn_ballot_w64(valid) == 0) dma4(g, ln.sink);
         } else {
             *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) =
                 load8(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
@@ -263,6 +284,27 @@ __device__ __forceinline__ u32x4 lds_a_transposed(const elem_t* slab, int c, int
     // rows krow and krow + 8 share their swizzle (it depends on row mod 8 only)
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 8 * HD));
+    u32x2 l2 = __builtin_bit_cast(u32x2, lo);
+    u32x2 h2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 r = {l2[0], l2[1], h2[0], h2[1]};
+    return r;
+}
+
+// The same transposed A operand with its eight k positions in natural order (slab rows
+// 16c + 8hf + {0..7}), to pair with a B operand read row-major from LDS rather than taken from an
+// accumulator.
+template <int HD>
+__device__ __forceinline__ u32x4 lds_a_transposed_nat(const elem_t* slab, int c, int d0, int lane) {
+    const int hf = lane >> 5;
+    const int i16 = lane & 15;
+    const int xb = lane & 16;
+    const int krow = 16 * c + 8 * hf + (i16 >> 2);
+    const int e = d0 + xb + 4 * (i16 & 3);
+    const elem_t* p0 = slab + krow * HD + (((e >> 3) ^ swz<HD>(krow)) << 3) + (e & 7);
+    const elem_t* p1 = slab + (krow + 4) * HD + (((e >> 3) ^ swz<HD>(krow + 4)) << 3) + (e & 7);
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo);
     u32x2 h2 = __builtin_bit_cast(u32x2, hi);
     u32x4 r = {l2[0], l2[1], h2[0], h2[1]};

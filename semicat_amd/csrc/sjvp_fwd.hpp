@@ -35,7 +35,8 @@ struct FwdSmem {
     static constexpr int nt = JVP ? 4 : 2;                      // tensors per stage
     static constexpr int slot = nt * Slab<HD>::elems;            // elements per ring slot
     static constexpr int own = DMA ? (JVP ? 2 : 1) * kWaves * Slab<HD>::elems : 0;
-    static constexpr int bytes = (own + R * slot) * (int)sizeof(elem_t);
+    static constexpr int sink = (own + R * slot) * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSinkBytes;
     static_assert(!DMA || R * slot >= kWaves * StoreStage<HD>::elems, "ring too small to stage stores");
 };
 
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid);
+    ln.init(tid, smem_raw + SM::sink);
     const int qrow = qb * kOwned + wave * 32 + x;  // the query this lane owns
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;

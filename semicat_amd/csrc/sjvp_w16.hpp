@@ -1,0 +1,222 @@
+// Building blocks of the 16-wide kernels (gfx950): eight wavefronts per workgroup, each owning 16
+// positions of the owned axis, so that a wavefront's accumulators and operands stay well below 128
+// registers and two to four wavefronts share a SIMD (their MFMA, VALU and LDS phases overlap).
+//
+// Tile algebra (v_mfma_f32_16x16x32_{bf16,f16}): C[y][x] += sum_k A[y][k] B[k][x] with
+//     A: lane l holds row y = l % 16, k = 8*(l/16) + i (i < 8);   B: column x = l % 16, same k;
+//     C: lane l holds column x = l % 16 and, in register j < 4, row y = 4*(l/16) + j.
+// The owned side is the B operand (registers), the looped side the A operand (row-major LDS reads).
+// A stage of 32 looped rows gives two 16-row score tiles t = 0, 1; converted to 16-bit, their eight
+// registers are directly the B operand of the next contraction OUT^T[d][x] += A'[d][y] Tile[y][x]
+// under the k numbering  k = 8g + i  <->  y = 16*(i/4) + 4g + i%4  (g = l/16), and A' in that numbering
+// is what two transposing LDS reads (rows 4g..4g+3 and 16+4g..16+4g+3, sixteen columns) deliver.
+#pragma once
+#include "sjvp_device.hpp"
+
+namespace sjvp {
+
+constexpr int kWaves16 = 8;
+constexpr int kThreads16 = 64 * kWaves16;
+constexpr int kOwned16 = 16 * kWaves16;  // owned positions per workgroup (== kOwned)
+constexpr int kSink16 = 16;              // bytes of LDS that placeholder copies may overwrite
+static_assert(kOwned16 == kOwned, "both kernel families use the same workgroup grid");
+
+struct Src {
+    const elem_t* ptr;  // [L][D] slice of one (batch, head)
+    int64_t sl;         // row stride in elements
+};
+
+// Per-thread geometry of an LDS-DMA copy of NS slabs that lie back to back in LDS: slab j holds rows
+// 32*(j % SPTN) .. +31 (relative to the first row of the copy window) of tensor j / SPTN.  Successive
+// calls of issue() copy successive windows (32*SPTN rows further down every tensor).  Every wave
+// issues exactly N vector-memory instructions per call: a wave with no valid lane issues a 4-byte
+// placeholder copy into the sink, which keeps the vmcnt arithmetic of wait_stages exact.
+template <int HD, int NS, int SPTN>
+struct CopyPlan {
+    static constexpr int chunks = Slab<HD>::chunks;
+    static constexpr int total = NS * chunks;
+    static constexpr int N = (total + kThreads16 - 1) / kThreads16;
+    static constexpr int NTENS = NS / SPTN;
+    static_assert(NS % SPTN == 0 && chunks % 64 == 0, "slabs are whole multiples of a wave's 64 chunks");
+    const elem_t* src[N];  // global address of this thread's chunk in the next window
+    int64_t adv[N];        // elements from one window to the next (wave-uniform)
+    int row[N];            // row of the chunk relative to the window's first row
+    uint32_t wbase[N];     // byte offset of the wave's first chunk position from the region base
+    uint32_t pos[N];       // byte offset of this thread's chunk position
+    bool ok[N];            // the column of the chunk is below D
+    bool on[N];            // the position exists (wave-uniform)
+    const elem_t* any;     // some valid global address (source of placeholder copies)
+    uint32_t sink;
+
+    // Tensors are passed one by one (not as an array) so that the wave-uniform choice among them
+    // stays a chain of scalar selects.
+    __device__ __forceinline__ void init(int tid, int first_row, int D, const void* sink_lds, Src t0,
+                                         Src t1 = Src{nullptr, 0}, Src t2 = Src{nullptr, 0},
+                                         Src t3 = Src{nullptr, 0}, Src t4 = Src{nullptr, 0},
+                                         Src t5 = Src{nullptr, 0}) {
+        static_assert(NTENS <= 6, "at most six tensors per copy");
+        constexpr int CH = HD / 8;
+        any = t0.ptr;
+        sink = lds_addr(sink_lds);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const int p = tid + i * kThreads16;
+            on[i] = p < total;
+            const int j = p / chunks, q = p % chunks;
+            const int r = q / CH;
+            const int c8 = 8 * ((q % CH) ^ swz<HD>(r));
+            const int tensor = __builtin_amdgcn_readfirstlane(j / SPTN);
+            const elem_t* ptr = t0.ptr;
+            int64_t sl = t0.sl;
+            auto pick = [&](int k, const Src& t) {
+                if (k < NTENS && tensor == k) {
+                    ptr = t.ptr;
+                    sl = t.sl;
+                }
+            };
+            pick(1, t1);
+            pick(2, t2);
+            pick(3, t3);
+            pick(4, t4);
+            pick(5, t5);
+            row[i] = 32 * (j % SPTN) + r;
+            src[i] = ptr + (int64_t)(first_row + row[i]) * sl + c8;
+            adv[i] = 32 * SPTN * sl;
+            ok[i] = c8 < D;
+            wbase[i] = (uint32_t)((p & ~63) * 16);
+            pos[i] = (uint32_t)(p * 16);
+        }
+    }
+
+    // Copy the next window into `region`; rows_left = rows of the window that exist (zero fill beyond).
+    __device__ __forceinline__ void issue(elem_t* region, int rows_left) {
+        const uint32_t base = lds_addr(region);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            bool valid = false;
+            if (total % kThreads16 == 0 || on[i]) {
+                valid = ok[i] && row[i] < rows_left;
+                if (valid) {
+                    dma16(src[i], base + wbase[i]);
+                } else {
+                    *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(region) + pos[i]) =
+                        u32x4{0u, 0u, 0u, 0u};
+                }
+                src[i] += adv[i];
+            }
+            if (__builtin_amdgcn_ballot_w64(valid) == 0) {
+                if ((threadIdx.x & 63) == 0) dma4(any, sink);
+            }
+        }
+    }
+};
+
+// A operand of a score tile: rows 16t .. 16t+15 of a slab, k = head-dimension chunk c of 32.
+template <int HD>
+__device__ __forceinline__ u32x4 lds_a_rows16(const elem_t* slab, int t, int c, int n, int g) {
+    const int r = 16 * t + n;
+    return *reinterpret_cast<const u32x4*>(slab + r * HD + (((4 * c + g) ^ swz<HD>(r)) << 3));
+}
+
+// B operands of one owned row (all head-dimension chunks of 32) from a landed slab.
+template <int HD>
+__device__ __forceinline__ void read_b_operands16(u32x4* out, const elem_t* slab, int r, int g) {
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c)
+        out[c] = *reinterpret_cast<const u32x4*>(slab + r * HD + (((4 * c + g) ^ swz<HD>(r)) << 3));
+}
+
+// A' operand of an output contraction: A'[d0 + n][k] for the lane group's eight slab rows
+// 4g..4g+3 and 16+4g..16+4g+3 (see the k numbering at the top).  Two ds_read_b64_tr_b16: within a
+// group of 16 lanes, lane 4j+c supplies the address of row (first + j), columns 4c..4c+3, and lane i
+// receives column i of those four rows.  Rows r and r+16 share their swizzle.
+template <int HD>
+__device__ __forceinline__ u32x4 lds_a_tr16(const elem_t* slab, int d0, int lane) {
+    const int g = lane >> 4;
+    const int i16 = lane & 15;
+    const int r = 4 * g + (i16 >> 2);
+    const int e = d0 + 4 * (i16 & 3);
+    const elem_t* p0 = slab + r * HD + (((e >> 3) ^ swz<HD>(r)) << 3) + (e & 7);
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 16 * HD));
+    u32x2 l2 = __builtin_bit_cast(u32x2, lo);
+    u32x2 h2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
+    return out;
+}
+
+// The same with its eight k positions in natural order: slab rows first + 8g + {0..7}
+// (pairs with a B operand read row-major from LDS).
+template <int HD>
+__device__ __forceinline__ u32x4 lds_a_tr16_nat(const elem_t* slab, int first, int d0, int lane) {
+    const int g = lane >> 4;
+    const int i16 = lane & 15;
+    const int r = first + 8 * g + (i16 >> 2);
+    const int e = d0 + 4 * (i16 & 3);
+    const elem_t* p0 = slab + r * HD + (((e >> 3) ^ swz<HD>(r)) << 3) + (e & 7);
+    const elem_t* p1 = slab + (r + 4) * HD + (((e >> 3) ^ swz<HD>(r + 4)) << 3) + (e & 7);
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
+    u32x2 l2 = __builtin_bit_cast(u32x2, lo);
+    u32x2 h2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
+    return out;
+}
+
+// The two score-like tiles of a stage as the B operand of the next contraction.
+template <typename T>
+__device__ __forceinline__ u32x4 pack_b16(const f32x4& t0, const f32x4& t1) {
+    u32x4 r = {T::pack2(t0[0], t0[1]), T::pack2(t0[2], t0[3]), T::pack2(t1[0], t1[1]),
+               T::pack2(t1[2], t1[3])};
+    return r;
+}
+
+// Sum / maximum over the four lanes (l, l^16, l^32, l^48) that share an owned position.
+__device__ __forceinline__ float group_sum(float v) {
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+__device__ __forceinline__ float group_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+// Per-wave staging tile of the coalesced row stores: [16 rows][HD + 8] elements.
+template <int HD>
+struct StoreStage16 {
+    static constexpr int pitch = HD + 8;
+    static constexpr int elems = 16 * pitch;
+};
+
+// Store OUT[row0 + r][0..D) for r < 16 from transposed accumulator tiles acc[HD/16] (lane = row,
+// registers = 4 consecutive columns 16*dt + 4g ..) scaled by mul: 8-byte writes into the wave's
+// staging tile, 16-byte reads back row-major, 16-byte global stores (a 128-byte row per 8 lanes).
+// Issues exactly max(1, HD / 32) global store instructions.
+template <typename T, int HD>
+__device__ __forceinline__ void store_tile16(elem_t* stage, elem_t* gp, int64_t sl, int row0, int L, int D,
+                                             const f32x4* acc, float mul, int lane) {
+    constexpr int P = StoreStage16<HD>::pitch;
+    const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) {
+        u32x2 val = {T::pack2(acc[dt][0] * mul, acc[dt][1] * mul), T::pack2(acc[dt][2] * mul, acc[dt][3] * mul)};
+        *reinterpret_cast<u32x2*>(stage + n * P + 16 * dt + 4 * g) = val;
+    }
+    constexpr int CH = HD / 8;    // 16-byte chunks per row
+    constexpr int RPI = 64 / CH;  // rows per store instruction
+#pragma unroll
+    for (int it = 0; it < (16 + RPI - 1) / RPI; ++it) {
+        const int r = it * RPI + lane / CH;
+        const int c = lane % CH;
+        if (RPI <= 16 || r < 16) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * P + 8 * c);
+            if (row0 + r < L && 8 * c < D) *reinterpret_cast<u32x4*>(gp + (int64_t)(row0 + r) * sl + 8 * c) = v;
+        }
+    }
+}
+
+}  // namespace sjvp
