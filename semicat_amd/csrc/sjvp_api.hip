@@ -7,6 +7,7 @@
 
 #include "sjvp_bwd.hpp"
 #include "sjvp_bwd_fused.hpp"
+#include "sjvp_bwd16.hpp"
 #include "sjvp_fwd.hpp"
 #include "sjvp_fwd16.hpp"
 
@@ -81,7 +82,7 @@ int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
 #define SJVP_F16_R 2
 #endif
 #ifndef SJVP_F16_OCC
-#define SJVP_F16_OCC 2
+#define SJVP_F16_OCC 4
 #endif
 template <typename T, int HD>
 int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
@@ -121,8 +122,13 @@ int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         // short key axis: one launch, one workgroup per (batch, head)
         if (parts == SJVP_BWD_ALL && p.Lk <= kOwned) {
             constexpr int FR = Ring<HD>::fused;
+#ifdef SJVP_FUSED32
             return launch(bwd_fused_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
                           FusedSmem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p);
+#else
+            return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
+                          Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
+#endif
         }
     }
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.

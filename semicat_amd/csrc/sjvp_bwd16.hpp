@@ -1,0 +1,353 @@
+// Single-launch attention-JVP backward, 16-wide form, for short key axes (Lk <= 128, head dimension
+// <= 64, 16-byte aligned rows): one workgroup of eight wavefronts per (batch, head) owns every key
+// (16 per wavefront), streams the queries once in stages of 32 and produces all six gradients, so
+// each of the sixteen tensors crosses HBM exactly once and every score-side tile is computed once.
+//
+// Mathematics as in sjvp_bwd.hpp.  Per stage of 32 queries:
+//   1. threads 0..255: row sums s4, s7d of the NEXT stage from its G, dO, O, TO slabs (8 per row);
+//   2. wave w (keys 16w..16w+15): tiles S, S_dot, W, XY -> P, P_dot, dS_dot, dS (queries in
+//      registers, keys in lanes); dK, dV, dK_dot, dV_dot accumulate in registers; dS and dS_dot go
+//      as 16-bit into an LDS bounce tile [key][query];
+//   3. after a barrier, wave w forms one 16x16 tile of dQ and one of dQ_dot for the stage from the
+//      bounce tile and the own rows of K, K_dot (both through transposing LDS reads) and stores
+//      them: a stage's dQ rows are complete after one pass over the keys, so nothing is accumulated
+//      across stages and no atomics or partial sums are needed.
+// Results are deterministic.
+#pragma once
+#include "sjvp_bwd.hpp"
+#include "sjvp_w16.hpp"
+
+namespace sjvp {
+
+// LDS layout: [own K, K_dot: four slabs each][own V, V_dot: four slabs each; once they have been
+// read into registers the same memory is the bounce tile dS (, dS_dot): [128 keys][32 queries + pad]]
+// [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d][sink]
+// After the last stage the ring doubles as the per-wave staging tiles of the output stores.
+template <int HD, int R, bool HAS_DO, bool HAS_G>
+struct Fused16Smem {
+    static constexpr int nt = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
+    static constexpr int stat_elems = 6 * kStageRows * 2;  // 6 float arrays of 32, in elem_t units
+    static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
+    static constexpr int own_k = (HAS_G ? 2 : 1) * 4 * Slab<HD>::elems;  // K (, K_dot)
+    static constexpr int own_v = own_k;                                  // V (, V_dot)
+    static constexpr int bpitch = 48;  // elements per key row: 4 rows of a transposing read hit distinct banks
+    static constexpr int bounce_one = kOwned16 * bpitch;
+    static constexpr int bounce = (HAS_G ? 2 : 1) * bounce_one;
+    static constexpr int vregion = own_v > bounce ? own_v : bounce;
+    static constexpr int sink = (own_k + vregion + R * slot) * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSink16;
+    static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
+};
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G>
+__global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdParams p) {
+    static_assert(HD <= 64, "the accumulators of four gradients must fit the register file");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    using SM = Fused16Smem<HD, R, HAS_DO, HAS_G>;
+    constexpr int SE = Slab<HD>::elems;
+    elem_t* ownK = reinterpret_cast<elem_t*>(smem_raw);  // K slabs 0..3, then K_dot slabs 0..3
+    elem_t* ownV = ownK + SM::own_k;                      // V slabs 0..3, then V_dot slabs 0..3
+    elem_t* bounceS = ownV;                               // aliases V, V_dot after the prologue
+    elem_t* bounceT = ownV + SM::bounce_one;
+    elem_t* ring = ownV + SM::vregion;
+    // slot layout
+    constexpr int oTQ = SE, oG = 2 * SE, oDO = (HAS_G ? 3 : 1) * SE;
+    constexpr int oO = oDO + (HAS_DO ? SE : 0), oTO = oO + SE;
+    constexpr int oST = SM::nt * SE;
+    constexpr int BP = SM::bpitch;
+    constexpr int KC = HD / 32;
+    constexpr int DT = HD / 16;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int bh = blockIdx.x;
+    const int b = bh / p.H, h = bh % p.H;
+    const int key_slabs = (p.Lk + 31) >> 5;           // 32-key slabs that hold at least one key
+    const bool wave_active = (wave >> 1) < key_slabs;  // waves of a partly filled slab all take part
+
+    // own rows first (they land first), then the ring
+    {
+        CopyPlan<HD, HAS_G ? 16 : 8, 4> own_plan;
+        if constexpr (HAS_G)
+            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
+                          Src{p.tk.head(b, h), p.tk.sl}, Src{p.v.head(b, h), p.v.sl},
+                          Src{p.tv.head(b, h), p.tv.sl});
+        else
+            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
+                          Src{p.v.head(b, h), p.v.sl});
+        own_plan.issue(ownK, p.Lk);
+    }
+    using StagePlan = CopyPlan<HD, SM::nt, 1>;
+    constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
+    StagePlan plan;
+    {
+        const Src q{p.q.head(b, h), p.q.sl}, o{p.o.head(b, h), p.o.sl};
+        if constexpr (HAS_G && HAS_DO)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl}, o,
+                      Src{p.to.head(b, h), p.to.sl});
+        else if constexpr (HAS_G)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl}, o, Src{p.to.head(b, h), p.to.sl});
+        else
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl}, o);
+    }
+    const int ns = (p.Lq + kStageRows - 1) / kStageRows;
+    int issued = 0;
+    auto issue_next = [&]() {
+        elem_t* slot = ring + (issued % R) * SM::slot;
+        const int row0 = issued * kStageRows;
+        plan.issue(slot, p.Lq - row0);
+        // raw lse (wave 0) and mu (wave 1) of the stage's rows (rows < Lr exist); every wave issues
+        // exactly one 4-byte LDS-DMA instruction, the others as a placeholder into the sink
+        float* raw = reinterpret_cast<float*>(slot + oST);
+        if (wave < 2) {
+            const float* src = (wave == 1 && HAS_G) ? p.mu : p.lse;
+            if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(raw) + (uint32_t)(wave * 32 * 4));
+        } else {
+            if (lane == 0) dma4(plan.any, plan.sink);
+        }
+        ++issued;
+    };
+    while (issued < R && issued < ns) issue_next();
+    const float sl2 = p.scale * kLog2e;
+
+    // Row sums of a landed stage: thread t < 256 handles row t/8, columns 8*(t%8) .. +7; the eight
+    // partial sums meet through lane shuffles and the thread of column 0 writes the row's statistics.
+    auto row_sums = [&](elem_t* slot) {
+        if (tid >= 256) return;
+        const int r = tid >> 3, part = tid & 7;
+        float s4 = 0.f, s7d = 0.f;
+        if (part < HD / 8) {
+            const int off = r * HD + ((part ^ swz<HD>(r)) << 3);
+            const u32x4 o4 = *reinterpret_cast<const u32x4*>(slot + oO + off);
+            u32x4 g4, t4, d4;
+            if constexpr (HAS_G) {
+                g4 = *reinterpret_cast<const u32x4*>(slot + oG + off);
+                t4 = *reinterpret_cast<const u32x4*>(slot + oTO + off);
+            }
+            if constexpr (HAS_DO) d4 = *reinterpret_cast<const u32x4*>(slot + oDO + off);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float o0 = T::to_float((elem_t)(o4[i] & 0xffffu));
+                const float o1 = T::to_float((elem_t)(o4[i] >> 16));
+                if constexpr (HAS_G) {
+                    const float g0 = T::to_float((elem_t)(g4[i] & 0xffffu));
+                    const float g1 = T::to_float((elem_t)(g4[i] >> 16));
+                    const float t0 = T::to_float((elem_t)(t4[i] & 0xffffu));
+                    const float t1 = T::to_float((elem_t)(t4[i] >> 16));
+                    s4 += g0 * o0 + g1 * o1;
+                    s7d += g0 * t0 + g1 * t1;
+                }
+                if constexpr (HAS_DO) {
+                    const float d0 = T::to_float((elem_t)(d4[i] & 0xffffu));
+                    const float d1 = T::to_float((elem_t)(d4[i] >> 16));
+                    s7d += d0 * o0 + d1 * o1;
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 1; m < 8; m <<= 1) {
+            s4 += __shfl_xor(s4, m, 64);
+            s7d += __shfl_xor(s7d, m, 64);
+        }
+        if (part == 0) {
+            float* raw = reinterpret_cast<float*>(slot + oST);
+            float* fin = raw + 2 * kStageRows;
+            fin[0 * kStageRows + r] = raw[r] * kLog2e;
+            fin[1 * kStageRows + r] = HAS_G ? raw[kStageRows + r] : 0.f;
+            fin[2 * kStageRows + r] = s4;
+            fin[3 * kStageRows + r] = s7d;
+        }
+    };
+
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    f32x4 dk[DT], dv[DT], dtk[DT], dtv[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        dk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // Step 2: this wave's 32 x 16 tiles of one stage.
+    auto tile = [&](const elem_t* slot) {
+        const elem_t* sQ = slot;
+        const elem_t* sTQ = slot + oTQ;
+        const elem_t* sG = slot + oG;
+        const elem_t* sDO = slot + oDO;
+        const float* sStat = reinterpret_cast<const float*>(slot + oST) + 2 * kStageRows;
+        f32x4 s[2], ts[2], w[2], xy[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                const u32x4 aq = lds_a_rows16<HD>(sQ, t, c, n, g);
+                s[t] = T::mfma16(aq, kB[c], s[t]);
+                if constexpr (HAS_G) {
+                    ts[t] = T::mfma16(aq, tkB[c], ts[t]);
+                    const u32x4 atq = lds_a_rows16<HD>(sTQ, t, c, n, g);
+                    ts[t] = T::mfma16(atq, kB[c], ts[t]);
+                    const u32x4 ag = lds_a_rows16<HD>(sG, t, c, n, g);
+                    w[t] = T::mfma16(ag, vB[c], w[t]);
+                    xy[t] = T::mfma16(ag, tvB[c], xy[t]);
+                }
+                if constexpr (HAS_DO) {
+                    const u32x4 ado = lds_a_rows16<HD>(sDO, t, c, n, g);
+                    xy[t] = T::mfma16(ado, vB[c], xy[t]);
+                }
+            }
+        }
+        // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (register j of tile t is query 16t + 4g + j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int r0 = 16 * t + 4 * g;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+            const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+            const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+            const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
+                s[t][j] = pj;
+                if constexpr (HAS_G) {
+                    const float nn = fmaf(ts[t][j], p.scale, -mu4[j]);
+                    const float dts = pj * (w[t][j] - s44[j]);
+                    w[t][j] = dts;
+                    xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[j]));
+                    ts[t][j] = pj * nn;
+                } else {
+                    xy[t][j] = pj * (xy[t][j] - s74[j]);
+                }
+            }
+        }
+        const u32x4 pB = pack_b16<T>(s[0], s[1]);
+        const u32x4 dsB = pack_b16<T>(xy[0], xy[1]);
+        u32x4 pdB, dtsB;
+        if constexpr (HAS_G) {
+            pdB = pack_b16<T>(ts[0], ts[1]);
+            dtsB = pack_b16<T>(w[0], w[1]);
+        }
+        // bounce[key][query]: the packed registers 2t, 2t+1 are queries 16t + 4g .. + 3 of key 16w + n
+        {
+            elem_t* bs = bounceS + (wave * 16 + n) * BP + 4 * g;
+            *reinterpret_cast<u32x2*>(bs) = u32x2{dsB[0], dsB[1]};
+            *reinterpret_cast<u32x2*>(bs + 16) = u32x2{dsB[2], dsB[3]};
+            if constexpr (HAS_G) {
+                elem_t* bt = bounceT + (wave * 16 + n) * BP + 4 * g;
+                *reinterpret_cast<u32x2*>(bt) = u32x2{dtsB[0], dtsB[1]};
+                *reinterpret_cast<u32x2*>(bt + 16) = u32x2{dtsB[2], dtsB[3]};
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            const u32x4 aq = lds_a_tr16<HD>(sQ, 16 * d, lane);
+            dk[d] = T::mfma16(aq, dsB, dk[d]);
+            if constexpr (HAS_G) {
+                dtk[d] = T::mfma16(aq, dtsB, dtk[d]);
+                const u32x4 atq = lds_a_tr16<HD>(sTQ, 16 * d, lane);
+                dk[d] = T::mfma16(atq, dtsB, dk[d]);
+                const u32x4 ag = lds_a_tr16<HD>(sG, 16 * d, lane);
+                dtv[d] = T::mfma16(ag, pB, dtv[d]);
+                dv[d] = T::mfma16(ag, pdB, dv[d]);
+            }
+            if constexpr (HAS_DO) {
+                const u32x4 ado = lds_a_tr16<HD>(sDO, 16 * d, lane);
+                dv[d] = T::mfma16(ado, pB, dv[d]);
+            }
+        }
+    };
+
+    // B operand of step 3: Tile[k = key][x = query 16*qt + n] from a bounce tile, keys of slab kk in
+    // the k numbering of lds_a_tr16 (rows 4g..4g+3 and 16+4g..16+4g+3 of the slab).
+    auto bounce_b = [&](const elem_t* bounce, int kk, int qt) {
+        const int i16 = lane & 15;
+        const elem_t* p0 = bounce + (32 * kk + 4 * g + (i16 >> 2)) * BP + 16 * qt + 4 * (i16 & 3);
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 16 * BP));
+        u32x2 l2 = __builtin_bit_cast(u32x2, lo);
+        u32x2 h2 = __builtin_bit_cast(u32x2, hi);
+        return u32x4{l2[0], l2[1], h2[0], h2[1]};
+    };
+
+    // Step 3: 16 x 16 tiles (head-dimension tile dt, query tile qt) of dQ and dQ_dot for the stage.
+    // HD = 64: wave w forms tile w of both; HD = 32: waves 0..3 form dQ, waves 4..7 dQ_dot.
+    constexpr int NTILES = 2 * DT;
+    auto row_outputs = [&](int row0) {
+#pragma unroll
+        for (int which = 0; which < (HAS_G ? 2 : 1); ++which) {
+            const int tile_id = NTILES == 8 ? wave : wave - 4 * which;
+            if (tile_id < 0 || tile_id >= NTILES) continue;
+            const int dt = tile_id % DT, qt = tile_id / DT;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int kk = 0; kk < key_slabs; ++kk) {
+                const u32x4 ak = lds_a_tr16<HD>(ownK + kk * SE, 16 * dt, lane);
+                if (which == 0) {
+                    acc = T::mfma16(ak, bounce_b(bounceS, kk, qt), acc);
+                    if constexpr (HAS_G) {
+                        const u32x4 atk = lds_a_tr16<HD>(ownK + (4 + kk) * SE, 16 * dt, lane);
+                        acc = T::mfma16(atk, bounce_b(bounceT, kk, qt), acc);
+                    }
+                } else {
+                    acc = T::mfma16(ak, bounce_b(bounceT, kk, qt), acc);
+                }
+            }
+            // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3
+            const int qrow = row0 + 16 * qt + n;
+            const int col = 16 * dt + 4 * g;
+            if (qrow < p.Lq && col < p.D) {
+                const OutView& t = which == 0 ? p.dq : p.dtq;
+                u32x2 val = {T::pack2(acc[0] * p.scale, acc[1] * p.scale),
+                             T::pack2(acc[2] * p.scale, acc[3] * p.scale)};
+                *reinterpret_cast<u32x2*>(t.head(b, h) + (int64_t)qrow * t.sl + col) = val;
+            }
+        }
+    };
+
+    wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
+    __syncthreads();
+    {
+        const int r = 16 * (wave & 1) + n;
+        const int sidx = wave >> 1;
+        read_b_operands16<HD>(kB, ownK + sidx * SE, r, g);
+        read_b_operands16<HD>(vB, ownV + sidx * SE, r, g);
+        if constexpr (HAS_G) {
+            read_b_operands16<HD>(tkB, ownK + (4 + sidx) * SE, r, g);
+            read_b_operands16<HD>(tvB, ownV + (4 + sidx) * SE, r, g);
+        }
+    }
+    row_sums(ring);
+    for (int i = 0; i < ns; ++i) {
+        // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
+        // every wave has read V, V_dot, whose memory the bounce tile takes over)
+        __syncthreads();
+        if (i >= 1 && issued < ns) issue_next();
+        elem_t* slot = ring + (i % R) * SM::slot;
+        if (wave_active) tile(slot);
+        if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
+        __syncthreads();
+        if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
+        row_outputs(i * kStageRows);
+    }
+    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    if (!wave_active) return;
+    elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
+    const int row0 = wave * 16;
+    store_tile16<T, HD>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane);
+    if constexpr (HAS_G)
+        store_tile16<T, HD>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane);
+    store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
+    if constexpr (HAS_G)
+        store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
+}
+
+}  // namespace sjvp
