@@ -95,6 +95,14 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         else
             plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl}, o);
     }
+#ifdef SJVP_X_STAMP
+    float st_v[40];
+    int st_n = 0;
+    const unsigned long long t_0 = __builtin_amdgcn_s_memtime();
+#define BSTAMP() do { st_v[st_n++] = (float)(long long)(__builtin_amdgcn_s_memtime() - t_0); } while (0)
+#else
+#define BSTAMP() do {} while (0)
+#endif
     const int ns = (p.Lq + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
@@ -149,11 +157,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
                 }
             }
         }
-#pragma unroll
-        for (int m = 1; m < 8; m <<= 1) {
-            s4 += __shfl_xor(s4, m, 64);
-            s7d += __shfl_xor(s7d, m, 64);
-        }
+        s4 = sum8(s4);
+        s7d = sum8(s7d);
         if (part == 0) {
             float* raw = reinterpret_cast<float*>(slot + oST);
             float* fin = raw + 2 * kStageRows;
@@ -282,39 +287,57 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // Step 3: 16 x 16 tiles (head-dimension tile dt, query tile qt) of dQ and dQ_dot for the stage.
     // HD = 64: wave w forms tile w of both; HD = 32: waves 0..3 form dQ, waves 4..7 dQ_dot.
     constexpr int NTILES = 2 * DT;
-    auto row_outputs = [&](int row0) {
-#pragma unroll
-        for (int which = 0; which < (HAS_G ? 2 : 1); ++which) {
-            const int tile_id = NTILES == 8 ? wave : wave - 4 * which;
-            if (tile_id < 0 || tile_id >= NTILES) continue;
-            const int dt = tile_id % DT, qt = tile_id / DT;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int kk = 0; kk < key_slabs; ++kk) {
-                const u32x4 ak = lds_a_tr16<HD>(ownK + kk * SE, 16 * dt, lane);
-                if (which == 0) {
-                    acc = T::mfma16(ak, bounce_b(bounceS, kk, qt), acc);
-                    if constexpr (HAS_G) {
-                        const u32x4 atk = lds_a_tr16<HD>(ownK + (4 + kk) * SE, 16 * dt, lane);
-                        acc = T::mfma16(atk, bounce_b(bounceT, kk, qt), acc);
-                    }
-                } else {
-                    acc = T::mfma16(ak, bounce_b(bounceT, kk, qt), acc);
+    auto row_outputs = [&](int row0, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;  // all four key slabs hold keys
+        const int tq = wave;                           // dQ tile of this wave
+        const int tt = NTILES == 8 ? wave : wave - 4;      // dQ_dot tile of this wave
+        const bool do_q = tq < NTILES;
+        const bool do_t = HAS_G && tt >= 0 && tt < NTILES;
+        const int tile_id = do_q ? tq : tt;
+        if (!do_q && !do_t) return;
+        const int dt = tile_id % DT, qt = tile_id / DT;
+        // three independent chains: dS K, dS_dot K_dot (both into dQ) and dS_dot K (dQ_dot)
+        f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
+        auto step = [&](int kk) {
+            const u32x4 ak = lds_a_tr16<HD>(ownK + kk * SE, 16 * dt, lane);
+            if (do_q) {
+                a0 = T::mfma16(ak, bounce_b(bounceS, kk, qt), a0);
+                if constexpr (HAS_G) {
+                    const u32x4 bt = bounce_b(bounceT, kk, qt);
+                    const u32x4 atk = lds_a_tr16<HD>(ownK + (4 + kk) * SE, 16 * dt, lane);
+                    a1 = T::mfma16(atk, bt, a1);
+                    if (do_t) a2 = T::mfma16(ak, bt, a2);
                 }
+            } else {
+                a2 = T::mfma16(ak, bounce_b(bounceT, kk, qt), a2);
             }
-            // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3
-            const int qrow = row0 + 16 * qt + n;
-            const int col = 16 * dt + 4 * g;
-            if (qrow < p.Lq && col < p.D) {
-                const OutView& t = which == 0 ? p.dq : p.dtq;
-                u32x2 val = {T::pack2(acc[0] * p.scale, acc[1] * p.scale),
-                             T::pack2(acc[2] * p.scale, acc[3] * p.scale)};
-                *reinterpret_cast<u32x2*>(t.head(b, h) + (int64_t)qrow * t.sl + col) = val;
+        };
+        if constexpr (FULL) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) step(kk);
+        } else {
+            for (int kk = 0; kk < key_slabs; ++kk) step(kk);
+        }
+        // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3
+        const int qrow = row0 + 16 * qt + n;
+        const int col = 16 * dt + 4 * g;
+        if (qrow < p.Lq && col < p.D) {
+            if (do_q) {
+                a0 += a1;
+                u32x2 val = {T::pack2(a0[0] * p.scale, a0[1] * p.scale), T::pack2(a0[2] * p.scale, a0[3] * p.scale)};
+                *reinterpret_cast<u32x2*>(p.dq.head(b, h) + (int64_t)qrow * p.dq.sl + col) = val;
+            }
+            if (do_t) {
+                u32x2 val = {T::pack2(a2[0] * p.scale, a2[1] * p.scale), T::pack2(a2[2] * p.scale, a2[3] * p.scale)};
+                *reinterpret_cast<u32x2*>(p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl + col) = val;
             }
         }
     };
 
+    BSTAMP();
     wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
     __syncthreads();
+    BSTAMP();
     {
         const int r = 16 * (wave & 1) + n;
         const int sidx = wave >> 1;
@@ -330,15 +353,23 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
         __syncthreads();
+        BSTAMP();
         if (i >= 1 && issued < ns) issue_next();
         elem_t* slot = ring + (i % R) * SM::slot;
+        BSTAMP();
         if (wave_active) tile(slot);
+        BSTAMP();
         if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
         __syncthreads();
+        BSTAMP();
         if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
-        row_outputs(i * kStageRows);
+        BSTAMP();
+        if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
+        else row_outputs(i * kStageRows, std::false_type{});
+        BSTAMP();
     }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    BSTAMP();
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = wave * 16;
@@ -348,6 +379,15 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
     if constexpr (HAS_G)
         store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
+#ifdef SJVP_X_STAMP
+    BSTAMP();
+    __builtin_amdgcn_s_waitcnt(0);
+    BSTAMP();
+    if (tid == SJVP_X_STAMP * 64) {
+        p.lse2[(int64_t)bh * p.Lr] = (float)(t_0 & 0xffffffull);
+        for (int k = 0; k < st_n; ++k) p.lse2[(int64_t)bh * p.Lr + 1 + k] = st_v[k];
+    }
+#endif
 }
 
 }  // namespace sjvp

@@ -185,6 +185,16 @@ __device__ __forceinline__ float group_max(float v) {
     return v;
 }
 
+// Sum over each aligned group of eight consecutive lanes, by DPP moves (no LDS traffic): the quad
+// permutations [1,0,3,2] and [2,3,0,1], then row_half_mirror, which pairs lane i with lane 7 - i of
+// its group of eight, i.e. with the other quad.
+__device__ __forceinline__ float sum8(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
 // Per-wave staging tile of the coalesced row stores: [16 rows][HD + 8] elements.
 template <int HD>
 struct StoreStage16 {
