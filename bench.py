@@ -30,11 +30,10 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
-# kernel of --calib-copy).
+# kernel of --calib-copy: one FETCH_SIZE unit is 2 KiB, one WRITE_SIZE unit 1 KiB there).
 MEASURED_TRAFFIC_BYTES = {
-    "fwd_kernel": (2 * 37004.0 + 25344.0) * 1024,      # FETCH_SIZE counts 2 KiB per unit on the copy
-    "bwd_row_kernel": (2 * 61983.0 + 25728.0) * 1024,  # kernel (131089 for 262144 KiB), WRITE_SIZE 1 KiB
-    "bwd_col_kernel": (2 * 50090.5 + 49152.0) * 1024,
+    "fwd16_kernel": (2 * 36937.6 + 25344.0) * 1024,
+    "bwd_fused16_kernel": (2 * 61933.1 + 73728.0) * 1024,
 }
 
 
@@ -166,8 +165,6 @@ def main() -> int:
             return e0.elapsed_time(e1) / n  # ms
 
         fwd_ms = timed(fwd)
-        row_ms = timed(lambda: bwd(_lib.SJVP_BWD_ROW))
-        col_ms = timed(lambda: bwd(_lib.SJVP_BWD_COL))
         bwd_ms = timed(bwd)
 
         if a.calib_copy:
@@ -181,16 +178,15 @@ def main() -> int:
     ms_per_step = wall / a.steps * 1e3
     tflops = step_flops() / (ms_per_step * 1e-3) / 1e12
 
-    # Algorithmic work per (batch, head), e = 2 bytes.  The backward's 15 contractions and 16 tensor
-    # passes are credited once: the column-owned launch gets the 6 recomputed score-side contractions
-    # and its 6 output contractions (24 L^2 D flop) and the 8 tensors it reads plus the 4 it writes;
-    # the row-owned launch gets its 3 output contractions (6 L^2 D) and O, TO, dQ, dQ_dot (its second
-    # score-side pass and its re-read of the other eight inputs are redundant work, not credited).
+    # Algorithmic work per (batch, head), e = 2 bytes.  Forward: 6 tile contractions (12 L^2 D flop);
+    # it reads q, k, v and the three tangents and writes O, TO, lse, mu.  Backward: 15 contractions
+    # (30 L^2 D flop) in one launch; it reads those six, O, TO, dO, dTO, lse, mu and writes the six
+    # gradients: every tensor crosses HBM once.
     BH = B * H
     work = {
-        "fwd_kernel": {"ms": fwd_ms, "flops": 12.0 * BH * L * L * D, "bytes": BH * (8.0 * L * D * 2 + 8.0 * L)},
-        "bwd_row_kernel": {"ms": row_ms, "flops": 6.0 * BH * L * L * D, "bytes": BH * (4.0 * L * D * 2 + 12.0 * L)},
-        "bwd_col_kernel": {"ms": col_ms, "flops": 24.0 * BH * L * L * D, "bytes": BH * (12.0 * L * D * 2 + 16.0 * L)},
+        "fwd16_kernel": {"ms": fwd_ms, "flops": 12.0 * BH * L * L * D, "bytes": BH * (8.0 * L * D * 2 + 8.0 * L)},
+        "bwd_fused16_kernel": {"ms": bwd_ms, "flops": 30.0 * BH * L * L * D,
+                               "bytes": BH * (16.0 * L * D * 2 + 8.0 * L)},
     }
     for w in work.values():
         w["GBps"] = w["bytes"] / (w["ms"] * 1e-3) / 1e9

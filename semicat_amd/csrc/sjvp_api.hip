@@ -6,7 +6,6 @@
 #include <math.h>
 
 #include "sjvp_bwd.hpp"
-#include "sjvp_bwd_fused.hpp"
 #include "sjvp_bwd16.hpp"
 #include "sjvp_fwd.hpp"
 #include "sjvp_fwd16.hpp"
@@ -43,9 +42,9 @@ int check_common(int B, int H, int Lq, int Lk, int D, int dtype) {
     return SJVP_OK;
 }
 
-template <typename K>
-int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params,
-           int threads = kThreads) {
+template <typename K, typename... Extra>
+int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params, int threads,
+           Extra... extra) {
     if (smem_bytes > 64 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -54,8 +53,13 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
             return SJVP_ERR_LAUNCH;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem_bytes, stream, params);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem_bytes, stream, params, extra...);
     return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
+}
+
+template <typename K>
+int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params) {
+    return launch(kernel, grid, smem_bytes, stream, params, kThreads);
 }
 
 // Ring depths (stages of 32 rows in flight) per head-dimension class, sized to the LDS left beside
@@ -67,6 +71,8 @@ struct Ring {
     static constexpr int row = 3;
     static constexpr int col = HD == 128 ? 3 : 4;
     static constexpr int fused = 3;
+    static constexpr int fwd16 = 2;
+    static constexpr int fwd16_primal = 4;
 };
 
 template <typename T, int HD, bool DMA>
@@ -78,17 +84,13 @@ int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     return launch(fwd_kernel<T, HD, RP, false, DMA>, grid, FwdSmem<HD, RP, false, DMA>::bytes, stream, p);
 }
 
-#ifndef SJVP_F16_R
-#define SJVP_F16_R 2
-#endif
-#ifndef SJVP_F16_OCC
-#define SJVP_F16_OCC 4
-#endif
 template <typename T, int HD>
 int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    constexpr int R = HD == 128 ? 2 : SJVP_F16_R;
-    constexpr int RP = 4;
-    constexpr int OCC = HD == 128 ? 2 : SJVP_F16_OCC;
+    // two stages in flight and at most 128 registers: two workgroups (sixteen waves) share a CU, which
+    // overlaps one's copies with the other's arithmetic; HD = 128 needs the whole register budget
+    constexpr int R = Ring<HD>::fwd16;
+    constexpr int RP = Ring<HD>::fwd16_primal;
+    constexpr int OCC = HD == 128 ? 2 : 4;
     if (jvp)
         return launch(fwd16_kernel<T, HD, R, true, OCC>, grid, Fwd16Smem<HD, R, true>::bytes, stream, p,
                       kThreads16);
@@ -100,14 +102,9 @@ template <typename T>
 int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
     if (p.vec) {
-#ifndef SJVP_NO_F16
         if (p.D <= 32) return fwd16_hd<T, 32>(p, grid, jvp, stream);
         if (p.D <= 64) return fwd16_hd<T, 64>(p, grid, jvp, stream);
         return fwd16_hd<T, 128>(p, grid, jvp, stream);
-#endif
-        if (p.D <= 32) return fwd_hd<T, 32, true>(p, grid, jvp, stream);
-        if (p.D <= 64) return fwd_hd<T, 64, true>(p, grid, jvp, stream);
-        return fwd_hd<T, 128, true>(p, grid, jvp, stream);
     }
     if (p.D <= 32) return fwd_hd<T, 32, false>(p, grid, jvp, stream);
     if (p.D <= 64) return fwd_hd<T, 64, false>(p, grid, jvp, stream);
@@ -122,13 +119,8 @@ int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         // short key axis: one launch, one workgroup per (batch, head)
         if (parts == SJVP_BWD_ALL && p.Lk <= kOwned) {
             constexpr int FR = Ring<HD>::fused;
-#ifdef SJVP_FUSED32
-            return launch(bwd_fused_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
-                          FusedSmem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p);
-#else
             return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
                           Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
-#endif
         }
     }
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.

@@ -95,14 +95,6 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         else
             plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl}, o);
     }
-#ifdef SJVP_X_STAMP
-    float st_v[40];
-    int st_n = 0;
-    const unsigned long long t_0 = __builtin_amdgcn_s_memtime();
-#define BSTAMP() do { st_v[st_n++] = (float)(long long)(__builtin_amdgcn_s_memtime() - t_0); } while (0)
-#else
-#define BSTAMP() do {} while (0)
-#endif
     const int ns = (p.Lq + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
@@ -124,7 +116,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     const float sl2 = p.scale * kLog2e;
 
     // Row sums of a landed stage: thread t < 256 handles row t/8, columns 8*(t%8) .. +7; the eight
-    // partial sums meet through lane shuffles and the thread of column 0 writes the row's statistics.
+    // partial sums meet through DPP moves and the thread of column 0 writes the row's statistics.
     auto row_sums = [&](elem_t* slot) {
         if (tid >= 256) return;
         const int r = tid >> 3, part = tid & 7;
@@ -334,10 +326,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
     };
 
-    BSTAMP();
     wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
     __syncthreads();
-    BSTAMP();
     {
         const int r = 16 * (wave & 1) + n;
         const int sidx = wave >> 1;
@@ -353,23 +343,16 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
         __syncthreads();
-        BSTAMP();
-        if (i >= 1 && issued < ns) issue_next();
+            if (i >= 1 && issued < ns) issue_next();
         elem_t* slot = ring + (i % R) * SM::slot;
-        BSTAMP();
-        if (wave_active) tile(slot);
-        BSTAMP();
-        if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
+            if (wave_active) tile(slot);
+            if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
         __syncthreads();
-        BSTAMP();
-        if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
-        BSTAMP();
-        if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
+            if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
+            if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
         else row_outputs(i * kStageRows, std::false_type{});
-        BSTAMP();
-    }
+        }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
-    BSTAMP();
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = wave * 16;
@@ -379,15 +362,6 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
     if constexpr (HAS_G)
         store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
-#ifdef SJVP_X_STAMP
-    BSTAMP();
-    __builtin_amdgcn_s_waitcnt(0);
-    BSTAMP();
-    if (tid == SJVP_X_STAMP * 64) {
-        p.lse2[(int64_t)bh * p.Lr] = (float)(t_0 & 0xffffffull);
-        for (int k = 0; k < st_n; ++k) p.lse2[(int64_t)bh * p.Lr + 1 + k] = st_v[k];
-    }
-#endif
 }
 
 }  // namespace sjvp

@@ -156,8 +156,9 @@ struct Slab {
     static constexpr int per_thread = (chunks + kThreads - 1) / kThreads;
 };
 
+// LDS byte address of a pointer into shared memory: the low half of its flat address.
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
-    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+    return (uint32_t)(uintptr_t)p;
 }
 
 // LDS-DMA: each active lane copies 16 bytes from its global address to LDS byte address
@@ -284,27 +285,6 @@ __device__ __forceinline__ u32x4 lds_a_transposed(const elem_t* slab, int c, int
     // rows krow and krow + 8 share their swizzle (it depends on row mod 8 only)
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 8 * HD));
-    u32x2 l2 = __builtin_bit_cast(u32x2, lo);
-    u32x2 h2 = __builtin_bit_cast(u32x2, hi);
-    u32x4 r = {l2[0], l2[1], h2[0], h2[1]};
-    return r;
-}
-
-// The same transposed A operand with its eight k positions in natural order (slab rows
-// 16c + 8hf + {0..7}), to pair with a B operand read row-major from LDS rather than taken from an
-// accumulator.
-template <int HD>
-__device__ __forceinline__ u32x4 lds_a_transposed_nat(const elem_t* slab, int c, int d0, int lane) {
-    const int hf = lane >> 5;
-    const int i16 = lane & 15;
-    const int xb = lane & 16;
-    const int krow = 16 * c + 8 * hf + (i16 >> 2);
-    const int e = d0 + xb + 4 * (i16 & 3);
-    const elem_t* p0 = slab + krow * HD + (((e >> 3) ^ swz<HD>(krow)) << 3) + (e & 7);
-    const elem_t* p1 = slab + (krow + 4) * HD + (((e >> 3) ^ swz<HD>(krow + 4)) << 3) + (e & 7);
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo);
     u32x2 h2 = __builtin_bit_cast(u32x2, hi);
     u32x4 r = {l2[0], l2[1], h2[0], h2[1]};

@@ -12,12 +12,6 @@
 
 namespace sjvp {
 
-#ifndef SJVP_FENCE_MODE
-#define SJVP_FENCE_MODE 0
-#endif
-#define SJVP_FENCE_A do { if (SJVP_FENCE_MODE & 1) asm volatile("" ::: "memory"); } while (0)
-#define SJVP_FENCE_B(d) do { if ((SJVP_FENCE_MODE & 2) || ((SJVP_FENCE_MODE & 4) && ((d) & 1))) asm volatile("" ::: "memory"); } while (0)
-
 // LDS layout: [own: Q (, Q_dot) rows of the workgroup, four slabs each][ring: R slots of K, V
 // (, K_dot, V_dot) stage slabs][sink].  After the last stage the ring doubles as the per-wave
 // staging tiles of the output stores.
@@ -72,14 +66,6 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
                   Src{p.tk.head(b, h), p.tk.sl}, Src{p.tv.head(b, h), p.tv.sl});
     else
         plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl}, Src{p.v.head(b, h), p.v.sl});
-#ifdef SJVP_X_STAMP
-    float st_v[16];
-    int st_n = 0;
-    const unsigned long long t_0 = __builtin_amdgcn_s_memtime();
-#define STAMP() do { st_v[st_n++] = (float)(long long)(__builtin_amdgcn_s_memtime() - t_0); } while (0)
-#else
-#define STAMP() do {} while (0)
-#endif
     const int ns = (p.Lk + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
@@ -102,10 +88,8 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         tacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    STAMP();
     wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
     __syncthreads();
-    STAMP();
     u32x4 qB[KC], tqB[KC];
     {
         const int r = 16 * (wave & 1) + n;
@@ -133,7 +117,6 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
                     ts[t] = T::mfma16(at, qB[c], ts[t]);
                 }
             }
-            SJVP_FENCE_A;
         }
         if (k0 + kStageRows > p.Lk) {  // wave-uniform: only the last stage can be ragged
             // keys beyond Lk are zero rows in LDS (their S_dot is already 0)
@@ -184,7 +167,6 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
                 const u32x4 atv = lds_a_tr16<HD>(sTV, 16 * d, lane);
                 tacc[d] = T::mfma16(atv, pb, tacc[d]);
             }
-            SJVP_FENCE_B(d);
         }
     };
 
@@ -198,10 +180,8 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         const elem_t* slot = ring + (i % R) * SM::slot;
         const int k0 = i * kStageRows;
         compute(slot, k0);
-        STAMP();
-    }
+        }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
-    STAMP();
     const int64_t so = (int64_t)bh * p.Lr + qrow;
     if (!wave_active) {
         // All 16 rows of this wave lie beyond Lq: their statistic rows get the values a zero query
@@ -239,15 +219,6 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
     store_tile16<T, HD>(stage_tile, p.o.head(b, h), p.o.sl, row0, p.Lq, p.D, acc, inv_l, lane);
     if constexpr (JVP)
         store_tile16<T, HD>(stage_tile, p.to.head(b, h), p.to.sl, row0, p.Lq, p.D, tacc, inv_l, lane);
-#ifdef SJVP_X_STAMP
-    STAMP();
-    __builtin_amdgcn_s_waitcnt(0);
-    STAMP();
-    if (tid == 0) {
-        p.lse[(int64_t)bh * p.Lr] = (float)(t_0 & 0xffffffull);
-        for (int k = 0; k < st_n; ++k) p.lse[(int64_t)bh * p.Lr + 1 + k] = st_v[k];
-    }
-#endif
 }
 
 }  // namespace sjvp

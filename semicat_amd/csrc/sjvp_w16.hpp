@@ -29,13 +29,13 @@ struct Src {
 // Per-thread geometry of an LDS-DMA copy of NS slabs that lie back to back in LDS: slab j holds rows
 // 32*(j % SPTN) .. +31 (relative to the first row of the copy window) of tensor j / SPTN.  Successive
 // calls of issue() copy successive windows (32*SPTN rows further down every tensor).  Every wave
-// issues exactly N vector-memory instructions per call: a wave with no valid lane issues a 4-byte
+// that takes part issues exactly N vector-memory instructions per call: a wave with no valid lane issues a 4-byte
 // placeholder copy into the sink, which keeps the vmcnt arithmetic of wait_stages exact.
-template <int HD, int NS, int SPTN>
+template <int HD, int NS, int SPTN, int NT = kThreads16>
 struct CopyPlan {
     static constexpr int chunks = Slab<HD>::chunks;
     static constexpr int total = NS * chunks;
-    static constexpr int N = (total + kThreads16 - 1) / kThreads16;
+    static constexpr int N = (total + NT - 1) / NT;  // NT threads take part (tid = 0 .. NT-1)
     static constexpr int NTENS = NS / SPTN;
     static_assert(NS % SPTN == 0 && chunks % 64 == 0, "slabs are whole multiples of a wave's 64 chunks");
     const elem_t* src[N];  // global address of this thread's chunk in the next window
@@ -60,7 +60,7 @@ struct CopyPlan {
         sink = lds_addr(sink_lds);
 #pragma unroll
         for (int i = 0; i < N; ++i) {
-            const int p = tid + i * kThreads16;
+            const int p = tid + i * NT;
             on[i] = p < total;
             const int j = p / chunks, q = p % chunks;
             const int r = q / CH;
@@ -94,7 +94,7 @@ struct CopyPlan {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             bool valid = false;
-            if (total % kThreads16 == 0 || on[i]) {
+            if (total % NT == 0 || on[i]) {
                 valid = ok[i] && row[i] < rows_left;
                 if (valid) {
                     dma16(src[i], base + wbase[i]);
@@ -140,25 +140,6 @@ __device__ __forceinline__ u32x4 lds_a_tr16(const elem_t* slab, int d0, int lane
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 16 * HD));
-    u32x2 l2 = __builtin_bit_cast(u32x2, lo);
-    u32x2 h2 = __builtin_bit_cast(u32x2, hi);
-    u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
-    return out;
-}
-
-// The same with its eight k positions in natural order: slab rows first + 8g + {0..7}
-// (pairs with a B operand read row-major from LDS).
-template <int HD>
-__device__ __forceinline__ u32x4 lds_a_tr16_nat(const elem_t* slab, int first, int d0, int lane) {
-    const int g = lane >> 4;
-    const int i16 = lane & 15;
-    const int r = first + 8 * g + (i16 >> 2);
-    const int e = d0 + 4 * (i16 & 3);
-    const elem_t* p0 = slab + r * HD + (((e >> 3) ^ swz<HD>(r)) << 3) + (e & 7);
-    const elem_t* p1 = slab + (r + 4) * HD + (((e >> 3) ^ swz<HD>(r + 4)) << 3) + (e & 7);
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p1));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo);
     u32x2 h2 = __builtin_bit_cast(u32x2, hi);
     u32x4 out = {l2[0], l2[1], h2[0], h2[1]};
