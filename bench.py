@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention-JVP forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--no-cpu-baseline] [--calib-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--graph] [--no-cpu-baseline] [--calib-copy]
 
 A step is one pass of the hot path over one batch: the fused forward (O, TO, lse, mu) followed by
 the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
@@ -88,7 +88,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay a HIP graph of one step instead of launching through the C ABI every step")
+    ap.add_argument("--no-graph", action="store_true", help="(default behaviour; kept for old command lines)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device copy (reference point for rocprofv3 --pmc byte counters)")
@@ -117,24 +119,23 @@ def main() -> int:
     nbytes = _lib.load().sjvp_bwd_workspace_bytes(B, H, L, L, D, _lib.SJVP_BF16)
     workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
 
-    def fwd():
-        kernels.attention_jvp_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False)
-
-    def bwd(parts=_lib.SJVP_BWD_ALL):
-        kernels.attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads,
-                                       workspace=workspace, parts=parts)
-
-    def step():
-        fwd()
-        bwd()
-
     stream = torch.cuda.Stream()  # default priority; graph capture needs a non-default stream
     graph = None
     with torch.cuda.stream(stream):
+        # Planned launches: arguments validated and converted once, each call is one trip through the
+        # C ABI (sjvp_fwd, then sjvp_bwd) on this stream.
+        fwd, _ = kernels.plan_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False)
+        bwd, _ = kernels.plan_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads,
+                                       workspace=workspace)
+
+        def step():
+            fwd()
+            bwd()
+
         for _ in range(3):
             step()
         stream.synchronize()
-        if not a.no_graph:
+        if a.graph:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 step()
@@ -152,7 +153,7 @@ def main() -> int:
         wall = time.perf_counter() - t0
 
         # Per-kernel durations: HIP events on the launch stream around runs of one kernel launched
-        # alone (eager launches; every kernel sees the same buffers as in the timed steps).
+        # alone (every kernel sees the same buffers as in the timed steps).
         def timed(fn, n=100):
             for _ in range(10):
                 fn()
@@ -224,7 +225,8 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": "config 2: LM1B-shaped DiT attention JVP fwd+bwd, B=64 H=12 L=128 D=64, "
                                "bf16 in / fp32 acc, non-causal, both cotangents",
-                   "launch": "eager" if graph is None else "hip-graph replay of one fwd+bwd step",
+                   "launch": "one sjvp_fwd + one sjvp_bwd call per step" if graph is None
+                             else "hip-graph replay of one fwd+bwd step",
                    "flop_model": "42*B*H*L^2*D"},
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "fwd_ms": fwd_ms,

@@ -19,6 +19,10 @@
 
 namespace sjvp {
 
+#ifndef SJVP_SCHED_BARRIER
+#define SJVP_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0)
+#endif
+
 // LDS layout: [own K, K_dot: four slabs each][own V, V_dot: four slabs each; once they have been
 // read into registers the same memory is the bounce tile dS (, dS_dot): [128 keys][32 queries + pad]]
 // [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d][sink]
@@ -179,8 +183,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         const elem_t* sDO = slot + oDO;
         const float* sStat = reinterpret_cast<const float*>(slot + oST) + 2 * kStageRows;
         f32x4 s[2], ts[2], w[2], xy[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        auto scores = [&](int t) __attribute__((always_inline)) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -202,10 +205,9 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
                     xy[t] = T::mfma16(ado, vB[c], xy[t]);
                 }
             }
-        }
+        };
         // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (register j of tile t is query 16t + 4g + j)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        auto pointwise = [&](int t) __attribute__((always_inline)) {
             const int r0 = 16 * t + 4 * g;
             const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
             const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
@@ -225,7 +227,24 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
                     xy[t][j] = pj * (xy[t][j] - s74[j]);
                 }
             }
+        };
+        // the second tile's MFMA chains run under the first tile's pointwise arithmetic
+        scores(0);
+        SJVP_SCHED_BARRIER;
+        scores(1);
+        pointwise(0);
+        SJVP_SCHED_BARRIER;
+        // the first transposed operands of the output contractions are fetched under the second
+        // tile's pointwise arithmetic
+        const u32x4 aq0 = lds_a_tr16<HD>(sQ, 0, lane);
+        u32x4 atq0, ag0, ado0;
+        if constexpr (HAS_G) {
+            atq0 = lds_a_tr16<HD>(sTQ, 0, lane);
+            ag0 = lds_a_tr16<HD>(sG, 0, lane);
         }
+        if constexpr (HAS_DO) ado0 = lds_a_tr16<HD>(sDO, 0, lane);
+        SJVP_SCHED_BARRIER;
+        pointwise(1);
         const u32x4 pB = pack_b16<T>(s[0], s[1]);
         const u32x4 dsB = pack_b16<T>(xy[0], xy[1]);
         u32x4 pdB, dtsB;
@@ -246,18 +265,18 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
-            const u32x4 aq = lds_a_tr16<HD>(sQ, 16 * d, lane);
+            const u32x4 aq = d == 0 ? aq0 : lds_a_tr16<HD>(sQ, 16 * d, lane);
             dk[d] = T::mfma16(aq, dsB, dk[d]);
             if constexpr (HAS_G) {
                 dtk[d] = T::mfma16(aq, dtsB, dtk[d]);
-                const u32x4 atq = lds_a_tr16<HD>(sTQ, 16 * d, lane);
+                const u32x4 atq = d == 0 ? atq0 : lds_a_tr16<HD>(sTQ, 16 * d, lane);
                 dk[d] = T::mfma16(atq, dtsB, dk[d]);
-                const u32x4 ag = lds_a_tr16<HD>(sG, 16 * d, lane);
+                const u32x4 ag = d == 0 ? ag0 : lds_a_tr16<HD>(sG, 16 * d, lane);
                 dtv[d] = T::mfma16(ag, pB, dtv[d]);
                 dv[d] = T::mfma16(ag, pdB, dv[d]);
             }
             if constexpr (HAS_DO) {
-                const u32x4 ado = lds_a_tr16<HD>(sDO, 16 * d, lane);
+                const u32x4 ado = d == 0 ? ado0 : lds_a_tr16<HD>(sDO, 16 * d, lane);
                 dv[d] = T::mfma16(ado, pB, dv[d]);
             }
         }

@@ -28,6 +28,22 @@ def stat_rows(L: int) -> int:
     return ((L + 127) // 128) * 128
 
 
+class _Launch:
+    """A validated call of the C ABI with its arguments already converted: calling it enqueues the
+    kernels on the stream that was current when it was planned (a few microseconds of host time,
+    for loops that launch the same problem many times).  Keeps the tensors alive."""
+
+    __slots__ = ("_fn", "_args", "_keep")
+
+    def __init__(self, fn, args, keep):
+        self._fn, self._args, self._keep = fn, args, keep
+
+    def __call__(self) -> None:
+        rc = self._fn(*self._args)
+        if rc:
+            _lib.check(rc)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
@@ -69,7 +85,7 @@ def _stat(buf: Optional[torch.Tensor], name: str, B: int, H: int, Lr: int, devic
 
 
 def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=None, to=None,
-                          lse=None, mu=None, li=None, with_li: bool = True
+                          lse=None, mu=None, li=None, with_li: bool = True, _plan: bool = False
                           ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                      Optional[torch.Tensor]]:
     """Fused forward on [B,H,L,D] views: returns (o, to, lse, mu, li); any of them may be passed in
@@ -97,10 +113,12 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.sjvp_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(tq), _ptr(tk), _ptr(tv), _ptr(o), _ptr(to),
-                          _ptr(lse), _ptr(mu), _ptr(li), B, H, Lq, Lk, D,
-                          _strides((q, k, v, tq, tk, tv, o, to)),
-                          float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+        args = (_ptr(q), _ptr(k), _ptr(v), _ptr(tq), _ptr(tk), _ptr(tv), _ptr(o), _ptr(to),
+                _ptr(lse), _ptr(mu), _ptr(li), B, H, Lq, Lk, D, _strides((q, k, v, tq, tk, tv, o, to)),
+                float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+        if _plan:
+            return _Launch(lib.sjvp_fwd, args, (q, k, v, tq, tk, tv, o, to, lse, mu, li)), (o, to, lse, mu, li)
+        rc = lib.sjvp_fwd(*args)
     _lib.check(rc)
     return o, to, lse, mu, li
 
@@ -133,7 +151,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
 
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
                            scale: Optional[float] = None, grads=None, workspace=None,
-                           parts: int = _lib.SJVP_BWD_ALL):
+                           parts: int = _lib.SJVP_BWD_ALL, _plan: bool = False):
     """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
     Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
     tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
@@ -199,12 +217,26 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
     tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.sjvp_bwd_parts(int(parts), *(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
-                          *(_ptr(t) for t in tensors[10:]), _ptr(workspace), nbytes, B, H, Lq, Lk, D,
-                          _strides(tensors), float(scale) if scale else 0.0, dtype_tag,
-                          ctypes.c_void_p(stream))
+        args = (int(parts), *(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
+                *(_ptr(t) for t in tensors[10:]), _ptr(workspace), nbytes, B, H, Lq, Lk, D,
+                _strides(tensors), float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+        if _plan:
+            return (_Launch(lib.sjvp_bwd_parts, args, tensors + (lse, mu, workspace)),
+                    (dq, dk, dv, dtq, dtk, dtv))
+        rc = lib.sjvp_bwd_parts(*args)
     _lib.check(rc)
     return dq, dk, dv, dtq, dtk, dtv
+
+
+def plan_forward(*args, **kwargs):
+    """attention_jvp_forward with the launch deferred: returns (launch, (o, to, lse, mu, li)), where
+    launch() enqueues the forward on the stream current at planning time."""
+    return attention_jvp_forward(*args, _plan=True, **kwargs)
+
+
+def plan_backward(*args, **kwargs):
+    """attention_jvp_backward with the launch deferred: returns (launch, (dq, dk, dv, dtq, dtk, dtv))."""
+    return attention_jvp_backward(*args, _plan=True, **kwargs)
 
 
 # ------------------------------------------------------------------------------------------------

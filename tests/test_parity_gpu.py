@@ -268,3 +268,25 @@ def test_reference_signature_wrappers(K):
     with pytest.raises(ValueError):
         K.flash_attention_jvp_multihead_kernel_wrapper(*(d[n][..., :8] for n in
                                                          ("q", "k", "v", "tq", "tk", "tv")))
+
+
+def test_planned_launches_match_direct_calls(K):
+    """plan_forward / plan_backward enqueue exactly what the direct calls compute (bitwise), and can be
+    called repeatedly."""
+    x = orc.make_inputs(2, 3, 128, 128, 64, seed=11, primal_scale=0.5, tangent_scale=0.1,
+                        dtype=torch.bfloat16)
+    d = _dev(x)
+    o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    fwd, (o2, to2, lse2, mu2, li2) = K.plan_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"],
+                                                   with_li=False)
+    bwd, g2 = K.plan_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o2, to2, lse2, mu2,
+                              dO=d["dO"], dTO=d["dTO"])
+    assert li2 is None
+    for _ in range(3):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    for a, b in zip((o, to, lse, mu) + tuple(g), (o2, to2, lse2, mu2) + tuple(g2)):
+        assert torch.equal(a, b)
