@@ -7,6 +7,7 @@
 
 #include "sjvp_bwd.hpp"
 #include "sjvp_bwd16.hpp"
+#include "sjvp_bwd16x.hpp"
 #include "sjvp_fwd.hpp"
 #include "sjvp_fwd16.hpp"
 
@@ -121,6 +122,26 @@ int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
             constexpr int FR = Ring<HD>::fused;
             return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
                           Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
+        }
+    }
+    if constexpr (DMA) {
+        // 16-wide pair: the row-owned kernel first (besides dQ, dQ_dot it leaves the row sums in the
+        // workspace), then the column-owned one; workgroups of four waves own 64 positions
+        constexpr int XR = HD == 128 ? 2 : 3;
+        int rc = SJVP_OK;
+        if (parts & SJVP_BWD_ROW)
+            rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, (HD == 128 ? 2 : 3)>,
+                        BH * (p.Lr / kXOwned16), Row16Smem<HD, XR, HAS_G>::bytes, stream, p, kXThreads16);
+        if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
+        const int grid = BH * ((p.Lk + kXOwned16 - 1) / kXOwned16);
+        using CS = Col16Smem<HD, XR, HAS_DO, HAS_G>;
+        if constexpr (HD == 128) {
+            // two launches, each accumulating two of the four gradients (register budget)
+            rc = launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 1, 2>, grid, CS::bytes, stream, p, kXThreads16);
+            if (rc != SJVP_OK) return rc;
+            return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 2, 2>, grid, CS::bytes, stream, p, kXThreads16);
+        } else {
+            return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
         }
     }
     // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.

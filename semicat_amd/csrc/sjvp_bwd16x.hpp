@@ -1,0 +1,413 @@
+// Attention-JVP backward for key axes beyond one workgroup, 16-wide form (gfx950; inputs with 16-byte
+// aligned rows): the row-owned and column-owned pair of sjvp_bwd.hpp (same mathematics, same
+// workspace hand-over of lse*log2e, s4, s7d) with 16 owned positions per wavefront, so that several
+// wavefronts share a SIMD and a workgroup's copies overlap another's arithmetic.
+//   bwd_row16_kernel   4 waves x 16 queries; streams K, V (, K_dot, V_dot)        -> dQ (, dQ_dot)
+//   bwd_col16_kernel   4 waves x 16 keys;    streams Q (, Q_dot, G) (, dO) + stats -> dK, dV (, dK_dot, dV_dot)
+// (workgroups of four waves: at 160-200 registers two or three of them share a CU)
+// The owned rows are loaded straight into registers (each lane its own 16-byte pieces), the streamed
+// side goes through an LDS ring filled by LDS-DMA.  Each gradient is accumulated in fp32 registers by
+// exactly one wavefront and written once: deterministic, no atomics.
+#pragma once
+#include "sjvp_bwd.hpp"
+#include "sjvp_w16.hpp"
+
+namespace sjvp {
+
+constexpr int kXWaves16 = 4;
+constexpr int kXThreads16 = 64 * kXWaves16;
+constexpr int kXOwned16 = 16 * kXWaves16;  // owned positions per workgroup
+
+// B operands (all head-dimension chunks of 32) of one owned row, straight from global memory.
+template <int HD>
+__device__ __forceinline__ void load_b_operands16(u32x4* out, const elem_t* row, int g, int D, bool valid) {
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c) out[c] = load8(row, 32 * c + 8 * g, D, valid, true);
+}
+
+// sum over the 16-bit pairs of a[i]*b[i]
+template <typename T>
+__device__ __forceinline__ float dot8(const u32x4& a, const u32x4& b) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        s += T::to_float((elem_t)(a[i] & 0xffffu)) * T::to_float((elem_t)(b[i] & 0xffffu));
+        s += T::to_float((elem_t)(a[i] >> 16)) * T::to_float((elem_t)(b[i] >> 16));
+    }
+    return s;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Row-owned kernel.  LDS: [ring of K | V (| K_dot | V_dot) stages][sink]; the ring doubles as store
+// staging after the last stage.
+template <int HD, int R, bool HAS_G>
+struct Row16Smem {
+    static constexpr int nt = HAS_G ? 4 : 2;
+    static constexpr int slot = nt * Slab<HD>::elems;
+    static constexpr int sink = R * slot * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSink16;
+    static_assert(R * slot >= kXWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
+};
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC>
+__global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    using SM = Row16Smem<HD, R, HAS_G>;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    constexpr int SE = Slab<HD>::elems;
+    constexpr int KC = HD / 32;
+    constexpr int DT = HD / 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int q_blocks = p.Lr / kXOwned16;  // statistic rows up to Lr are all covered
+    const int bh = blockIdx.x / q_blocks;
+    const int qb = blockIdx.x % q_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const int q0 = qb * kXOwned16;
+    const int qrow = q0 + wave * 16 + n;
+    const bool qvalid = qrow < p.Lq;
+    const bool wave_active = (q0 + wave * 16) < p.Lq;
+
+    // the ring first, so that the copies stream while the own rows are fetched
+    using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
+    constexpr int SPT = StagePlan::N;
+    StagePlan plan;
+    if constexpr (HAS_G)
+        plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl}, Src{p.v.head(b, h), p.v.sl},
+                  Src{p.tk.head(b, h), p.tk.sl}, Src{p.tv.head(b, h), p.tv.sl});
+    else
+        plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl}, Src{p.v.head(b, h), p.v.sl});
+    const int ns = (p.Lk + kStageRows - 1) / kStageRows;
+    int issued = 0;
+    auto issue_next = [&]() {
+        plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows);
+        ++issued;
+    };
+    while (issued < R && issued < ns) issue_next();
+
+    // own rows as B operands; row sums s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O) from the
+    // lane's 16-byte pieces, combined over the four lanes of a query
+    u32x4 qB[KC], tqB[KC], gB[KC], doB[KC];
+    float s4 = 0.f, s7d = 0.f;
+    {
+        u32x4 oR[KC], toR[KC];
+        load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
+        load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
+        if constexpr (HAS_G) {
+            load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
+            load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
+            load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
+        }
+        if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            if constexpr (HAS_G) {
+                s4 += dot8<T>(gB[c], oR[c]);
+                s7d += dot8<T>(gB[c], toR[c]);
+            }
+            if constexpr (HAS_DO) s7d += dot8<T>(doB[c], oR[c]);
+        }
+        s4 = group_sum(s4);
+        s7d = group_sum(s7d);
+    }
+    const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
+    const float lse2 = p.lse[so] * kLog2e;
+    const float mu = HAS_G ? p.mu[so] : 0.f;
+    if (g == 0) {
+        // every row below Lr is written (zeros beyond Lq except lse2, which is finite): the
+        // column-owned kernel, which runs after this one, stages 32-row groups
+        p.lse2[so] = lse2;
+        p.s4[so] = s4;
+        p.s7d[so] = s7d;
+    }
+    const float sl2 = p.scale * kLog2e;
+    f32x4 dq[DT], dtq[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        dq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    auto compute = [&](const elem_t* slot, int k0) {
+        const elem_t* sK = slot;
+        const elem_t* sV = slot + SE;
+        const elem_t* sTK = slot + 2 * SE;
+        const elem_t* sTV = slot + 3 * SE;
+        // tiles: rows = keys (registers), columns = this wave's queries (lanes)
+        f32x4 s[2], ts[2], w[2], xy[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                const u32x4 ak = lds_a_rows16<HD>(sK, t, c, n, g);
+                const u32x4 av = lds_a_rows16<HD>(sV, t, c, n, g);
+                s[t] = T::mfma16(ak, qB[c], s[t]);
+                if constexpr (HAS_G) {
+                    ts[t] = T::mfma16(ak, tqB[c], ts[t]);
+                    const u32x4 atk = lds_a_rows16<HD>(sTK, t, c, n, g);
+                    ts[t] = T::mfma16(atk, qB[c], ts[t]);
+                    w[t] = T::mfma16(av, gB[c], w[t]);
+                    const u32x4 atv = lds_a_rows16<HD>(sTV, t, c, n, g);
+                    xy[t] = T::mfma16(atv, gB[c], xy[t]);
+                }
+                if constexpr (HAS_DO) xy[t] = T::mfma16(av, doB[c], xy[t]);
+            }
+        }
+        const bool ragged = k0 + kStageRows > p.Lk;  // wave-uniform: only the last stage
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float pj = fast_exp2(fmaf(s[t][j], sl2, -lse2));
+                // keys beyond Lk are zero rows; exp(-lse) may overflow when every real score is very
+                // negative, so their P is forced to zero
+                if (ragged && k0 + 16 * t + 4 * g + j >= p.Lk) pj = 0.f;
+                if constexpr (HAS_G) {
+                    const float nn = fmaf(ts[t][j], p.scale, -mu);
+                    const float dts = pj * (w[t][j] - s4);
+                    w[t][j] = dts;
+                    xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s7d));
+                } else {
+                    xy[t][j] = pj * (xy[t][j] - s7d);
+                }
+            }
+        }
+        const u32x4 dsB = pack_b16<T>(xy[0], xy[1]);
+        u32x4 dtsB;
+        if constexpr (HAS_G) dtsB = pack_b16<T>(w[0], w[1]);
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            const u32x4 ak = lds_a_tr16<HD>(sK, 16 * d, lane);
+            dq[d] = T::mfma16(ak, dsB, dq[d]);
+            if constexpr (HAS_G) {
+                dtq[d] = T::mfma16(ak, dtsB, dtq[d]);
+                const u32x4 atk = lds_a_tr16<HD>(sTK, 16 * d, lane);
+                dq[d] = T::mfma16(atk, dtsB, dq[d]);
+            }
+        }
+    };
+
+    for (int i = 0; i < ns; ++i) {
+        // copies issued after stage i: the later stages; anything else in flight (the own rows'
+        // loads, the statistics) only makes the wait stricter
+        wait_stages<SPT>(issued - 1 - i);
+        __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+        if (i > 0 && issued < ns) issue_next();
+        if (wave_active) compute(ring + (i % R) * SM::slot, i * kStageRows);
+    }
+    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    if (!wave_active) return;
+    elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
+    const int row0 = q0 + wave * 16;
+    store_tile16<T, HD>(stage_tile, p.dq.head(b, h), p.dq.sl, row0, p.Lq, p.D, dq, p.scale, lane);
+    if constexpr (HAS_G)
+        store_tile16<T, HD>(stage_tile, p.dtq.head(b, h), p.dtq.sl, row0, p.Lq, p.D, dtq, p.scale, lane);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Column-owned kernel: a workgroup of four waves owns 64 keys.  PART selects the gradients that are
+// accumulated: 3 all four (HD <= 64), 1 dK (, dK_dot), 2 dV (, dV_dot) (HD = 128 runs as two launches
+// to stay inside the register file).  LDS: [ring of Q | [Q_dot | G] | [dO] | lse2, mu, s4, s7d stages]
+// [sink]; the ring doubles as store staging after the last stage.
+template <int HD, int R, bool HAS_DO, bool HAS_G>
+struct Col16Smem {
+    static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
+    static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
+    static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
+    static constexpr int sink = R * slot * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSink16;
+    static_assert(R * slot >= kXWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
+};
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int PART, int OCC>
+__global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    using SM = Col16Smem<HD, R, HAS_DO, HAS_G>;
+    constexpr bool DO_K = (PART & 1) != 0, DO_V = (PART & 2) != 0;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    constexpr int SE = Slab<HD>::elems;
+    constexpr int oTQ = SE, oG = 2 * SE, oDO = (HAS_G ? 3 : 1) * SE, oST = SM::nt * SE;
+    constexpr int KC = HD / 32;
+    constexpr int DT = HD / 16;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int k_blocks = (p.Lk + kXOwned16 - 1) / kXOwned16;
+    const int bh = blockIdx.x / k_blocks;
+    const int kb = blockIdx.x % k_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const int key0 = kb * kXOwned16;
+    const int krow = key0 + wave * 16 + n;
+    const bool kvalid = krow < p.Lk;
+    const bool wave_active = (key0 + wave * 16) < p.Lk;
+
+    using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
+    constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
+    StagePlan plan;
+    {
+        const Src q{p.q.head(b, h), p.q.sl};
+        if constexpr (HAS_G && HAS_DO)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
+        else if constexpr (HAS_G)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl});
+        else
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
+    }
+    const int ns = (p.Lq + kStageRows - 1) / kStageRows;
+    int issued = 0;
+    auto issue_next = [&]() {
+        elem_t* slot = ring + (issued % R) * SM::slot;
+        const int row0 = issued * kStageRows;
+        plan.issue(slot, p.Lq - row0);
+        // the four statistic arrays (lse2, mu, s4, s7d) of the stage's rows, one per wave, 32 lanes
+        // each (rows < Lr exist in all of them); every wave issues exactly one 4-byte LDS-DMA
+        const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;
+        float* st = reinterpret_cast<float*>(slot + oST);
+        if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
+        ++issued;
+    };
+    while (issued < R && issued < ns) issue_next();
+
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
+    if constexpr (DO_K) load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
+    if constexpr (HAS_G) {
+        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
+        if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+    }
+    const float sl2 = p.scale * kLog2e;
+    f32x4 dk[DT], dv[DT], dtk[DT], dtv[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        dk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    auto compute = [&](const elem_t* slot) {
+        const elem_t* sQ = slot;
+        const elem_t* sTQ = slot + oTQ;
+        const elem_t* sG = slot + oG;
+        const elem_t* sDO = slot + oDO;
+        const float* sStat = reinterpret_cast<const float*>(slot + oST);
+        // tiles: rows = queries (registers), columns = this wave's keys (lanes)
+        f32x4 s[2], ts[2], w[2], xy[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                const u32x4 aq = lds_a_rows16<HD>(sQ, t, c, n, g);
+                s[t] = T::mfma16(aq, kB[c], s[t]);
+                if constexpr (HAS_G) {
+                    ts[t] = T::mfma16(aq, tkB[c], ts[t]);
+                    const u32x4 atq = lds_a_rows16<HD>(sTQ, t, c, n, g);
+                    ts[t] = T::mfma16(atq, kB[c], ts[t]);
+                    if constexpr (DO_K) {
+                        const u32x4 ag = lds_a_rows16<HD>(sG, t, c, n, g);
+                        w[t] = T::mfma16(ag, vB[c], w[t]);
+                        xy[t] = T::mfma16(ag, tvB[c], xy[t]);
+                    }
+                }
+                if constexpr (HAS_DO && DO_K) {
+                    const u32x4 ado = lds_a_rows16<HD>(sDO, t, c, n, g);
+                    xy[t] = T::mfma16(ado, vB[c], xy[t]);
+                }
+            }
+        }
+        // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (register j of tile t is query 16t + 4g + j;
+        // rows beyond Lq are zero rows of Q, Q_dot, G, dO with finite statistics: they contribute nothing)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int r0 = 16 * t + 4 * g;
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+            const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+            const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+            const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
+                s[t][j] = pj;
+                if constexpr (HAS_G) {
+                    const float nn = fmaf(ts[t][j], p.scale, -mu4[j]);
+                    if constexpr (DO_K) {
+                        const float dts = pj * (w[t][j] - s44[j]);
+                        w[t][j] = dts;
+                        xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[j]));
+                    }
+                    if constexpr (DO_V) ts[t][j] = pj * nn;
+                } else if constexpr (DO_K) {
+                    xy[t][j] = pj * (xy[t][j] - s74[j]);
+                }
+            }
+        }
+        u32x4 pB, dsB, pdB, dtsB;
+        if constexpr (DO_V) pB = pack_b16<T>(s[0], s[1]);
+        if constexpr (DO_K) dsB = pack_b16<T>(xy[0], xy[1]);
+        if constexpr (HAS_G) {
+            if constexpr (DO_V) pdB = pack_b16<T>(ts[0], ts[1]);
+            if constexpr (DO_K) dtsB = pack_b16<T>(w[0], w[1]);
+        }
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+            if constexpr (DO_K) {
+                const u32x4 aq = lds_a_tr16<HD>(sQ, 16 * d, lane);
+                dk[d] = T::mfma16(aq, dsB, dk[d]);
+                if constexpr (HAS_G) {
+                    dtk[d] = T::mfma16(aq, dtsB, dtk[d]);
+                    const u32x4 atq = lds_a_tr16<HD>(sTQ, 16 * d, lane);
+                    dk[d] = T::mfma16(atq, dtsB, dk[d]);
+                }
+            }
+            if constexpr (DO_V) {
+                if constexpr (HAS_G) {
+                    const u32x4 ag = lds_a_tr16<HD>(sG, 16 * d, lane);
+                    dtv[d] = T::mfma16(ag, pB, dtv[d]);
+                    dv[d] = T::mfma16(ag, pdB, dv[d]);
+                }
+                if constexpr (HAS_DO) {
+                    const u32x4 ado = lds_a_tr16<HD>(sDO, 16 * d, lane);
+                    dv[d] = T::mfma16(ado, pB, dv[d]);
+                }
+            }
+        }
+    };
+
+    for (int i = 0; i < ns; ++i) {
+        wait_stages<SPT>(issued - 1 - i);
+        __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+        if (i > 0 && issued < ns) issue_next();
+        if (wave_active) compute(ring + (i % R) * SM::slot);
+    }
+    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    if (!wave_active) return;
+    elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
+    const int row0 = key0 + wave * 16;
+    if constexpr (DO_K) {
+        store_tile16<T, HD>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane);
+        if constexpr (HAS_G)
+            store_tile16<T, HD>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane);
+    }
+    if constexpr (DO_V) {
+        store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
+        if constexpr (HAS_G)
+            store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
+    }
+}
+
+}  // namespace sjvp
