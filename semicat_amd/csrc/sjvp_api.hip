@@ -63,26 +63,21 @@ int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& p
     return launch(kernel, grid, smem_bytes, stream, params, kThreads);
 }
 
-// Ring depths (stages of 32 rows in flight) per head-dimension class, sized to the LDS left beside
-// the workgroup's own rows (160 KB per CU; the forward keeps two workgroups per CU resident).
+// Ring depths (stages of 32 rows in flight) of the 16-wide kernels per head-dimension class, sized
+// to the LDS a workgroup may take when several of them are to share the 160 KB of a CU.
 template <int HD>
 struct Ring {
-    static constexpr int fwd = HD == 128 ? 2 : 4;         // with tangents (four slabs per stage)
-    static constexpr int fwd_primal = 4;                  // primal only (two slabs per stage)
-    static constexpr int row = 3;
-    static constexpr int col = HD == 128 ? 3 : 4;
+    static constexpr int fwd16 = 2;                    // with tangents (four slabs per stage)
+    static constexpr int fwd16_primal = 4;             // primal only (two slabs per stage)
     static constexpr int fused = 3;
-    static constexpr int fwd16 = 2;
-    static constexpr int fwd16_primal = 4;
+    static constexpr int pair = HD == 128 ? 2 : 3;     // row-owned / column-owned backward pair
 };
 
-template <typename T, int HD, bool DMA>
+// 32-wide forward for inputs of any alignment (register-staged copies, one stage in LDS)
+template <typename T, int HD>
 int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    constexpr int R = DMA ? Ring<HD>::fwd : 1;
-    constexpr int RP = DMA ? Ring<HD>::fwd_primal : 1;
-    if (jvp)
-        return launch(fwd_kernel<T, HD, R, true, DMA>, grid, FwdSmem<HD, R, true, DMA>::bytes, stream, p);
-    return launch(fwd_kernel<T, HD, RP, false, DMA>, grid, FwdSmem<HD, RP, false, DMA>::bytes, stream, p);
+    if (jvp) return launch(fwd_kernel<T, HD, true>, grid, FwdSmem<HD, true>::bytes, stream, p);
+    return launch(fwd_kernel<T, HD, false>, grid, FwdSmem<HD, false>::bytes, stream, p);
 }
 
 template <typename T, int HD>
@@ -107,27 +102,25 @@ int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
         if (p.D <= 64) return fwd16_hd<T, 64>(p, grid, jvp, stream);
         return fwd16_hd<T, 128>(p, grid, jvp, stream);
     }
-    if (p.D <= 32) return fwd_hd<T, 32, false>(p, grid, jvp, stream);
-    if (p.D <= 64) return fwd_hd<T, 64, false>(p, grid, jvp, stream);
-    return fwd_hd<T, 128, false>(p, grid, jvp, stream);
+    if (p.D <= 32) return fwd_hd<T, 32>(p, grid, jvp, stream);
+    if (p.D <= 64) return fwd_hd<T, 64>(p, grid, jvp, stream);
+    return fwd_hd<T, 128>(p, grid, jvp, stream);
 }
 
 template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
 int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
-    constexpr int R = DMA ? Ring<HD>::row : 1;
-    constexpr int CR = DMA ? Ring<HD>::col : 1;
-    if constexpr (DMA && HD <= 64) {
-        // short key axis: one launch, one workgroup per (batch, head)
-        if (parts == SJVP_BWD_ALL && p.Lk <= kOwned) {
-            constexpr int FR = Ring<HD>::fused;
-            return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
-                          Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
-        }
-    }
     if constexpr (DMA) {
+        if constexpr (HD <= 64) {
+            // short key axis: one launch, one workgroup per (batch, head)
+            if (parts == SJVP_BWD_ALL && p.Lk <= kOwned16) {
+                constexpr int FR = Ring<HD>::fused;
+                return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
+                              Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
+            }
+        }
         // 16-wide pair: the row-owned kernel first (besides dQ, dQ_dot it leaves the row sums in the
         // workspace), then the column-owned one; workgroups of four waves own 64 positions
-        constexpr int XR = HD == 128 ? 2 : 3;
+        constexpr int XR = Ring<HD>::pair;
         int rc = SJVP_OK;
         if (parts & SJVP_BWD_ROW)
             rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, (HD == 128 ? 2 : 3)>,
@@ -143,25 +136,23 @@ int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         } else {
             return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
         }
-    }
-    // Row-owned kernel first: besides dQ, dQ_dot it leaves the row sums in the workspace.
-    int rc = SJVP_OK;
-    if (parts & SJVP_BWD_ROW)
-        rc = launch(bwd_row_kernel<T, HD, R, HAS_DO, HAS_G, DMA>, BH * p.q_blocks,
-                    RowSmem<HD, R, HAS_DO, HAS_G, DMA>::bytes, stream, p);
-    if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
-    const int col_grid = BH * p.k_blocks;
-    using SM = ColSmem<HD, CR, HAS_DO, HAS_G, DMA>;
-    if constexpr (HD == 128) {
-        // two launches, each accumulating half of the head dimension (register budget)
-        rc = launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 0, 2, DMA>, col_grid, SM::bytes,
-                    stream, p);
-        if (rc != SJVP_OK) return rc;
-        return launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 2, 2, DMA>, col_grid,
-                      SM::bytes, stream, p);
     } else {
-        return launch(bwd_col_kernel<T, HD, CR, HAS_DO, HAS_G, true, true, 0, HD / 32, DMA>, col_grid,
-                      SM::bytes, stream, p);
+        // 32-wide pair for inputs of any alignment, same order
+        int rc = SJVP_OK;
+        if (parts & SJVP_BWD_ROW)
+            rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G>, BH * p.q_blocks, RowSmem<HD, HAS_G>::bytes, stream, p);
+        if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
+        const int col_grid = BH * p.k_blocks;
+        using SM = ColSmem<HD, HAS_DO, HAS_G>;
+        if constexpr (HD == 128) {
+            // two launches, each accumulating half of the head dimension (register budget)
+            rc = launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 0, 2>, col_grid, SM::bytes, stream, p);
+            if (rc != SJVP_OK) return rc;
+            return launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 2, 2>, col_grid, SM::bytes, stream, p);
+        } else {
+            return launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 0, HD / 32>, col_grid, SM::bytes,
+                          stream, p);
+        }
     }
 }
 

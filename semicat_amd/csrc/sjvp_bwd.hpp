@@ -10,7 +10,10 @@
 //     dV_dot = P^T G            dV = P_dot^T G + P^T dO
 //     dK_dot = s dS_dot^T Q     dK = s (dS^T Q + dS_dot^T Q_dot)
 //     dQ_dot = s dS_dot K       dQ = s (dS K + dS_dot K_dot)
-// The reference spends eight launches and 35 tile contractions on this; here it is two launches:
+// The reference spends eight launches and 35 tile contractions on this.  This file holds the 32-wide
+// pair for inputs of any alignment (the streamed side is copied through registers into one LDS
+// stage); inputs with 16-byte aligned rows take the 16-wide kernels of sjvp_bwd16.hpp (one launch,
+// short key axes) and sjvp_bwd16x.hpp (the same pair as here).  Two launches:
 //   bwd_row_kernel   a wavefront owns 32 queries -> dQ, dQ_dot; it also forms s4 and s7d for its
 //                    rows from O, TO, dO, G (O(L*D) work instead of five contractions) and leaves
 //                    them, with lse in log2 units, in the workspace for
@@ -21,7 +24,6 @@
 #include <type_traits>
 
 #include "sjvp_device.hpp"
-#include "sjvp_stream.hpp"
 
 namespace sjvp {
 
@@ -42,37 +44,21 @@ struct BwdParams {
 // ---------------------------------------------------------------------------------------------
 // Row-owned kernel: dQ (and dQ_dot).  Tiles are transposed (rows = keys in registers, columns =
 // this wave's queries in lanes), so the row statistics are per-lane scalars.
-// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's rows of Q, O (, Q_dot, G, TO)
-// (, dO), one slab per wave each][lse and mu of those rows][ring of K, V (, K_dot, V_dot) stages]; the ring
-// doubles as store staging after the last stage.
-template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
+// LDS layout: one stage of K, V (, K_dot, V_dot) slabs.
+template <int HD, bool HAS_G>
 struct RowSmem {
-    static constexpr bool own_lds = DMA && HD <= 64;
     static constexpr int nt = HAS_G ? 4 : 2;
     static constexpr int slot = nt * Slab<HD>::elems;
-    static constexpr int n_own = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
-    static constexpr int own = own_lds ? n_own * kWaves * Slab<HD>::elems : 0;
-    static constexpr int stat = own_lds ? 2 * kOwned * 2 : 0;  // two float arrays, in elem_t units
-    static constexpr int sink = (own + stat + R * slot) * (int)sizeof(elem_t);
-    static constexpr int bytes = sink + kSinkBytes;
+    static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
+template <typename T, int HD, bool HAS_DO, bool HAS_G>
 __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = RowSmem<HD, R, HAS_DO, HAS_G, DMA>;
-    constexpr bool OWN_LDS = SM::own_lds;
-    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
-    float* own_stat = reinterpret_cast<float*>(own + SM::own);
-    elem_t* ring = own + SM::own + SM::stat;
-    // own tensor order: Q, O, [Q_dot, G, TO], [dO]
-    constexpr int oQ = 0, oO = kWaves * Slab<HD>::elems, oTQ = 2 * kWaves * Slab<HD>::elems,
-                  oG = 3 * kWaves * Slab<HD>::elems, oTO = 4 * kWaves * Slab<HD>::elems,
-                  oDO = (HAS_G ? 5 : 2) * kWaves * Slab<HD>::elems;
+    elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
 
     constexpr int KC = HD / 16;
     constexpr int DT = HD / 32;
-    constexpr int SPT = SM::nt * Slab<HD>::per_thread;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,7 +69,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid, smem_raw + SM::sink);
+    ln.init(tid);
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
@@ -91,28 +77,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     u32x4 qB[KC], tqB[KC], gB[KC], doB[KC], oR[KC], toR[KC];
     float lse2 = 0.f, mu = 0.f;
     const int64_t so = (int64_t)bh * p.Lr + qrow;
-    if constexpr (OWN_LDS) {
-        // coalesced LDS-DMA copies of the workgroup's own rows; they are read back as B operands
-        // after the first ring stages have been issued
-        const int r0 = qb * kOwned;
-        auto own_fill = [&](int off, const TensorView& t) {
-#pragma unroll
-            for (int s4 = 0; s4 < kWaves; ++s4)
-                fill_slab<HD, true>(ln, own + off + s4 * Slab<HD>::elems, t.head(b, h), t.sl, r0 + 32 * s4,
-                                    p.Lq, p.D, true);
-        };
-        own_fill(oQ, p.q);
-        own_fill(oO, p.o);
-        if constexpr (HAS_G) {
-            own_fill(oTQ, p.tq);
-            own_fill(oG, p.dTO);
-            own_fill(oTO, p.to);
-        }
-        if constexpr (HAS_DO) own_fill(oDO, p.dO);
-        // lse (lanes 0-31) and mu (lanes 32-63) of this wave's 32 rows; rows < Lr exist in both
-        const float* src = hf == 0 ? p.lse : p.mu;
-        if (HAS_G || hf == 0) dma4(src + so, lds_addr(own_stat) + (uint32_t)(wave * 64 * 4));
-    } else {
+    {
         const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
         const elem_t* op = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
 #pragma unroll
@@ -139,17 +104,6 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         // Per-lane row statistics; an invalid query lane uses zeros (finite P, results discarded).
         lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
         mu = (qvalid && HAS_G) ? p.mu[so] : 0.f;
-        if constexpr (DMA) {
-            // retire these loads before the first LDS-DMA copy so that wait_stages() only has the
-            // ring's traffic to count
-            asm volatile("" : "+v"(lse2), "+v"(mu));
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                asm volatile("" : "+v"(qB[c]), "+v"(oR[c]));
-                if constexpr (HAS_G) asm volatile("" : "+v"(tqB[c]), "+v"(gB[c]), "+v"(toR[c]));
-                if constexpr (HAS_DO) asm volatile("" : "+v"(doB[c]));
-            }
-        }
     }
 
     // s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O): each half-lane holds half of the row's
@@ -180,21 +134,20 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         s4 += other_half(s4);
         s7d += other_half(s7d);
     };
-    if constexpr (!OWN_LDS) row_sums();
+    row_sums();
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = HAS_G ? p.tk.head(b, h) : nullptr;
     const elem_t* tvg = HAS_G ? p.tv.head(b, h) : nullptr;
     const float sl2 = p.scale * kLog2e;
 
-    auto issue = [&](int stage) {
-        elem_t* slot = ring + (stage % R) * SM::slot;
-        const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(ln, slot, kg, p.k.sl, row0, p.Lk, p.D, vec);
-        fill_slab<HD, DMA>(ln, slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
+    auto fill = [&](int st) {
+        const int row0 = st * kStageRows;
+        fill_slab<HD>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD, DMA>(ln, slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
-            fill_slab<HD, DMA>(ln, slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -205,12 +158,12 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         if constexpr (HAS_G) dtq[t] = f32x16{0};
     }
 
-    auto compute = [&](const elem_t* slot, int k0, auto ragged_tag) {
+    auto compute = [&](int k0, auto ragged_tag) {
         constexpr bool RAGGED = decltype(ragged_tag)::value;
-        const elem_t* sK = slot;
-        const elem_t* sV = slot + Slab<HD>::elems;
-        const elem_t* sTK = slot + 2 * Slab<HD>::elems;
-        const elem_t* sTV = slot + 3 * Slab<HD>::elems;
+        const elem_t* sK = stage;
+        const elem_t* sV = stage + Slab<HD>::elems;
+        const elem_t* sTK = stage + 2 * Slab<HD>::elems;
+        const elem_t* sTV = stage + 3 * Slab<HD>::elems;
         f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
@@ -263,71 +216,29 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     };
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
-    if constexpr (DMA) {
-        int issued = 0;
-        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
-        if constexpr (OWN_LDS) {
-            wait_stages<SPT>(issued);  // the own rows were issued before these stages
-            __syncthreads();
-            const int sw = wave * Slab<HD>::elems;
-            read_b_operands<HD>(qB, own + oQ + sw, x, hf);
-            read_b_operands<HD>(oR, own + oO + sw, x, hf);
-            if constexpr (HAS_G) {
-                read_b_operands<HD>(tqB, own + oTQ + sw, x, hf);
-                read_b_operands<HD>(gB, own + oG + sw, x, hf);
-                read_b_operands<HD>(toR, own + oTO + sw, x, hf);
-            }
-            if constexpr (HAS_DO) read_b_operands<HD>(doB, own + oDO + sw, x, hf);
-            lse2 = own_stat[wave * 64 + x] * kLog2e;
-            if constexpr (HAS_G) mu = own_stat[wave * 64 + 32 + x];
-            row_sums();
-        }
-    }
-    if (hf == 0) {  // every row below Lr is written (zeros beyond Lq except lse2, which is finite):
-                    // the column-owned kernel, which runs after this one, stages 32-row groups
+    if (hf == 0) {  // every row below Lr is written (zeros beyond Lq): the column-owned kernel, which
+                    // runs after this one, stages 32-row groups
         p.lse2[so] = lse2;
         p.s4[so] = s4;
         p.s7d[so] = s7d;
     }
     for (int i = 0; i < n; ++i) {
-        if constexpr (DMA) {
-            wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
-            __syncthreads();
-            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-        } else {
-            __syncthreads();
-            issue(i);
-            __syncthreads();
-        }
+        __syncthreads();  // the previous stage is fully consumed
+        fill(i);
+        __syncthreads();
         if (!wave_active) continue;
-        const elem_t* slot = ring + (i % R) * SM::slot;
         const int k0 = i * kStageRows;
-        if (k0 + kStageRows > p.Lk) {
-            compute(slot, k0, std::true_type{});
-        } else {
-            compute(slot, k0, std::false_type{});
-        }
+        if (k0 + kStageRows > p.Lk) compute(k0, std::true_type{});
+        else compute(k0, std::false_type{});
     }
-    if constexpr (DMA) {
-        __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
-        if (!wave_active) return;
-        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
-        const int row0 = qb * kOwned + wave * 32;
-        store_tile_coalesced<T, HD>(stage_tile, p.dq.head(b, h), p.dq.sl, row0, p.Lq, p.D, dq, p.scale,
-                                    lane);
-        if constexpr (HAS_G)
-            store_tile_coalesced<T, HD>(stage_tile, p.dtq.head(b, h), p.dtq.sl, row0, p.Lq, p.D, dtq,
-                                        p.scale, lane);
-    } else {
-        if (!qvalid) return;
-        elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
+    if (!qvalid) return;
+    elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) store_acc<T>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
-        if constexpr (HAS_G) {
-            elem_t* dtqrow = p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl;
+    for (int d = 0; d < DT; ++d) store_acc<T>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
+    if constexpr (HAS_G) {
+        elem_t* dtqrow = p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl;
 #pragma unroll
-            for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
-        }
+        for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
     }
 }
 
@@ -335,30 +246,23 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
 // Column-owned kernel: a wavefront owns 32 keys and streams the queries.  DO_K selects dK (and
 // dK_dot), DO_V selects dV (and dV_dot); DT0/NDT select the 32-wide head-dimension tiles that are
 // accumulated (at HD = 128 the work is split to stay inside the register file).
-// LDS layout on the LDS-DMA path at HD <= 64: [own: the workgroup's rows of K, V (, K_dot, V_dot),
-// one slab per wave each][ring of Q (, Q_dot, G) (, dO) stages, each followed by its row statistics]; the
-// ring doubles as store staging after the last stage.
-template <int HD, int R, bool HAS_DO, bool HAS_G, bool DMA>
+// LDS layout: one stage of Q (, Q_dot, G) (, dO) slabs followed by the stage's row statistics
+// (lse2, mu, s4, s7d).
+template <int HD, bool HAS_DO, bool HAS_G>
 struct ColSmem {
-    static constexpr bool own_lds = DMA && HD <= 64;
     static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
     static constexpr int stat_elems = 4 * kStageRows * 2;  // 4 float arrays of 32, in elem_t units
     static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
-    static constexpr int own = own_lds ? (HAS_G ? 4 : 2) * kWaves * Slab<HD>::elems : 0;
-    static constexpr int sink = (own + R * slot) * (int)sizeof(elem_t);
-    static constexpr int bytes = sink + kSinkBytes;
+    static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT,
-          bool DMA>
+template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT>
 __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd_col_kernel(
     const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = ColSmem<HD, R, HAS_DO, HAS_G, DMA>;
-    constexpr bool OWN_LDS = SM::own_lds;
-    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
-    elem_t* ring = own + SM::own;
-    // own tensor order: K, V, [K_dot, V_dot];  slot layout: Q | [Q_dot | G] | [dO] | stats(lse2, mu, s4, s7d)
+    using SM = ColSmem<HD, HAS_DO, HAS_G>;
+    elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
+    // stage layout: Q | [Q_dot | G] | [dO] | stats(lse2, mu, s4, s7d)
     constexpr int oTQ = Slab<HD>::elems;
     constexpr int oG = 2 * Slab<HD>::elems;
     constexpr int oDO = (HAS_G ? 3 : 1) * Slab<HD>::elems;
@@ -375,30 +279,13 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid, smem_raw + SM::sink);
-    // LDS-DMA instructions per stage issued by every wave: the tensors plus one 4-byte copy of
-    // statistics
-    constexpr int SPT = SM::nt * Slab<HD>::per_thread + 1;
+    ln.init(tid);
     const int krow = kb * kOwned + wave * 32 + x;  // the key this lane owns
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (kb * kOwned + wave * 32) < p.Lk;
 
     u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    if constexpr (OWN_LDS) {
-        const int r0 = kb * kOwned;
-        auto own_fill = [&](int idx, const TensorView& t) {
-#pragma unroll
-            for (int s4 = 0; s4 < kWaves; ++s4)
-                fill_slab<HD, true>(ln, own + (kWaves * idx + s4) * Slab<HD>::elems, t.head(b, h), t.sl,
-                                    r0 + 32 * s4, p.Lk, p.D, true);
-        };
-        own_fill(0, p.k);
-        own_fill(1, p.v);
-        if constexpr (HAS_G) {
-            own_fill(2, p.tk);
-            own_fill(3, p.tv);
-        }
-    } else {
+    {
         const elem_t* kp = p.k.head(b, h) + (int64_t)krow * p.k.sl;
         const elem_t* vp = p.v.head(b, h) + (int64_t)krow * p.v.sl;
 #pragma unroll
@@ -415,17 +302,6 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
                 if constexpr (DO_K) tvB[c] = load8(tvp, 16 * c + 8 * hf, p.D, kvalid, vec);
             }
         }
-        if constexpr (DMA) {
-#pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                asm volatile("" : "+v"(kB[c]));
-                if constexpr (DO_K) asm volatile("" : "+v"(vB[c]));
-                if constexpr (HAS_G) {
-                    asm volatile("" : "+v"(tkB[c]));
-                    if constexpr (DO_K) asm volatile("" : "+v"(tvB[c]));
-                }
-            }
-        }
     }
     const elem_t* qg = p.q.head(b, h);
     const elem_t* tqg = HAS_G ? p.tq.head(b, h) : nullptr;
@@ -433,31 +309,25 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     const elem_t* dog = HAS_DO ? p.dO.head(b, h) : nullptr;
     const float sl2 = p.scale * kLog2e;
 
-    auto issue = [&](int stage) {
-        elem_t* slot = ring + (stage % R) * SM::slot;
-        const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(ln, slot, qg, p.q.sl, row0, p.Lq, p.D, vec);
+    auto fill = [&](int st) {
+        const int row0 = st * kStageRows;
+        fill_slab<HD>(ln, stage, qg, p.q.sl, row0, p.Lq, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD, DMA>(ln, slot + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec);
-            fill_slab<HD, DMA>(ln, slot + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec);
+            fill_slab<HD>(ln, stage + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec);
+            fill_slab<HD>(ln, stage + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec);
         }
-        if constexpr (HAS_DO) fill_slab<HD, DMA>(ln, slot + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec);
+        if constexpr (HAS_DO) fill_slab<HD>(ln, stage + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec);
         // Row statistics of the stage (rows < Lr are defined in all four arrays; rows beyond Lq
-        // hold finite values and multiply zero rows of Q, Q_dot, G, dO below).
-        float* st = reinterpret_cast<float*>(slot + oST);
+        // hold finite values and multiply zero rows of Q, Q_dot, G, dO below): the four arrays are
+        // dealt to the waves, 32 lanes each.
+        float* st_lds = reinterpret_cast<float*>(stage + oST);
         const int64_t so = (int64_t)bh * p.Lr + row0 + (lane & 31);
-        // the four arrays (lse2, mu, s4, s7d) are dealt to the waves, 32 lanes each; every wave
-        // issues exactly one 4-byte LDS-DMA instruction
         constexpr int APW = 4 / kWaves;  // arrays per wave
         const int arr = wave * APW + hf;
         if (hf < APW) {
             const float* src = arr == 0 ? p.lse2 : arr == 1 ? p.mu : arr == 2 ? p.s4 : p.s7d;
             if (arr == 1 && !HAS_G) src = p.s4;  // mu is not used without the tangent cotangent
-            if constexpr (DMA) {
-                dma4(src + so, lds_addr(st) + (uint32_t)(wave * APW * 32 * 4));
-            } else {
-                st[arr * 32 + (lane & 31)] = src[so];
-            }
+            st_lds[arr * 32 + (lane & 31)] = src[so];
         }
     };
 
@@ -472,12 +342,12 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
         }
     }
 
-    auto compute = [&](const elem_t* slot) {
-        const elem_t* sQ = slot;
-        const elem_t* sTQ = slot + oTQ;
-        const elem_t* sG = slot + oG;
-        const elem_t* sDO = slot + oDO;
-        const float* sStat = reinterpret_cast<const float*>(slot + oST);
+    auto compute = [&]() {
+        const elem_t* sQ = stage;
+        const elem_t* sTQ = stage + oTQ;
+        const elem_t* sG = stage + oG;
+        const elem_t* sDO = stage + oDO;
+        const float* sStat = reinterpret_cast<const float*>(stage + oST);
         // tiles: rows = queries (registers), columns = this wave's keys (lanes)
         f32x16 s = {0}, ts = {0}, w = {0}, xy = {0};
 #pragma unroll
@@ -562,55 +432,13 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
     };
 
     const int n = (p.Lq + kStageRows - 1) / kStageRows;
-    if constexpr (DMA) {
-        int issued = 0;
-        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
-        if constexpr (OWN_LDS) {
-            wait_stages<SPT>(issued);  // the own rows were issued before these stages
-            __syncthreads();
-            read_b_operands<HD>(kB, own + wave * Slab<HD>::elems, x, hf);
-            if constexpr (DO_K) read_b_operands<HD>(vB, own + (kWaves + wave) * Slab<HD>::elems, x, hf);
-            if constexpr (HAS_G) {
-                read_b_operands<HD>(tkB, own + (2 * kWaves + wave) * Slab<HD>::elems, x, hf);
-                if constexpr (DO_K)
-                    read_b_operands<HD>(tvB, own + (3 * kWaves + wave) * Slab<HD>::elems, x, hf);
-            }
-        }
-    }
     for (int i = 0; i < n; ++i) {
-        if constexpr (DMA) {
-            wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
-            __syncthreads();
-            if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-        } else {
-            __syncthreads();
-            issue(i);
-            __syncthreads();
-        }
-        if (!wave_active) continue;
-        compute(ring + (i % R) * SM::slot);
+        __syncthreads();  // the previous stage is fully consumed
+        fill(i);
+        __syncthreads();
+        if (wave_active) compute();
     }
-    if constexpr (DMA) {
-        __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
-        if (!wave_active) return;
-        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
-        const int row0 = kb * kOwned + wave * 32;
-        // NDT tiles starting at head-dimension tile DT0: the staging tile and the row pointers are
-        // offset by 32*DT0 columns, and the column bound is reduced accordingly
-        const int dcol = 32 * DT0;
-        auto put = [&](const OutView& t, const f32x16* acc, float mul) {
-            store_tile_coalesced<T, 32 * NDT>(stage_tile, t.head(b, h) + dcol, t.sl, row0, p.Lk,
-                                              p.D - dcol, acc, mul, lane);
-        };
-        if constexpr (DO_K) {
-            put(p.dk, dk, p.scale);
-            if constexpr (HAS_G) put(p.dtk, dtk, p.scale);
-        }
-        if constexpr (DO_V) {
-            put(p.dv, dv, 1.0f);
-            if constexpr (HAS_G) put(p.dtv, dtv, 1.0f);
-        }
-    } else {
+    {
         if (!kvalid) return;
         if constexpr (DO_K) {
             elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;

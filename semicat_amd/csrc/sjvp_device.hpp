@@ -1,7 +1,7 @@
 // Device-side building blocks shared by the attention-JVP kernels (gfx950 / CDNA4 only).
 //
-// Tile algebra used everywhere in this library
-// --------------------------------------------
+// Tile algebra used everywhere in this library (32-wide form; sjvp_w16.hpp has the 16-wide one)
+// ------------------------------------------------------------------------------------------------
 // One wavefront (64 lanes) owns 32 positions of one sequence axis ("owned" axis X: queries in the
 // forward and in the dQ kernel, keys in the dK/dV kernel) and walks over the other axis ("looped"
 // axis Y) in stages of 32 rows.  Every score-like 32x32 tile is produced by
@@ -17,14 +17,14 @@
 //
 // Streaming
 // ---------
-// The looped side is streamed through a ring of LDS slots.  On the fast path the copy is done by
-// the LDS-DMA form of the global load (global_load_lds_dwordx4: 16 bytes per lane straight into
-// LDS, no registers), issued several stages ahead and retired with explicit s_waitcnt vmcnt(n), so
-// that HBM traffic overlaps the MFMA work of earlier stages.  A stage slab is unpadded ([32][HD]
-// 16-bit) and XOR-swizzled in units of 16 bytes, which keeps both LDS access patterns (row-major
-// 16-byte reads of 8 consecutive rows, and the 4-row x 32-byte footprint of a transposing read)
-// free of bank conflicts; because every lane of an LDS-DMA load supplies its own global address,
-// the swizzle costs nothing at copy time.
+// The looped side lives in LDS stage slabs: unpadded [32][HD] 16-bit, XOR-swizzled in units of 16
+// bytes, which keeps both LDS access patterns (row-major 16-byte reads, and the 4-row x 32-byte
+// footprint of a transposing read) free of bank conflicts.  The 16-wide kernels fill a ring of such
+// stages with the LDS-DMA form of the global load (global_load_lds_dwordx4: 16 bytes per lane
+// straight into LDS, no registers), issued ahead of use and retired with explicit
+// s_waitcnt vmcnt(n); because every lane of an LDS-DMA load supplies its own global address, the
+// swizzle costs nothing at copy time.  The 32-wide kernels (inputs of any alignment) copy one
+// stage at a time through registers.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -204,22 +204,17 @@ __device__ __forceinline__ void wait_stages(int ahead) {
 #undef SJVP_VMCNT
 }
 
-// Every shared-memory layout ends with this many bytes that LDS-DMA placeholders may overwrite.
-constexpr int kSinkBytes = 256;
-
-// Per-thread geometry of a slab copy: which 16-byte chunk positions of a slab this thread fills and
-// which (row, column) of the source they hold.  Computed once per kernel.
+// Per-thread geometry of a synchronous slab copy by the kThreads threads of a 32-wide workgroup:
+// which 16-byte chunk positions of a slab this thread fills and which (row, column) of the source
+// they hold.  Computed once per kernel.
 template <int HD>
 struct SlabLane {
     static constexpr int N = Slab<HD>::per_thread;
-    int r[N];        // slab row
-    int c8[N];       // source column (elements) of the chunk
-    int pos8[N];     // element offset of the chunk position inside the slab
-    uint32_t wbase[N];  // byte offset, inside the slab, of the wave's first chunk position
-    bool on[N];      // the position exists (slabs smaller than the workgroup)
-    uint32_t sink;   // LDS byte address of kSinkBytes that nothing reads
-    __device__ __forceinline__ void init(int tid, const void* sink_lds) {
-        sink = lds_addr(sink_lds);
+    int r[N];     // slab row
+    int c8[N];    // source column (elements) of the chunk
+    int pos8[N];  // element offset of the chunk position inside the slab
+    bool on[N];   // the position exists (slabs smaller than the workgroup)
+    __device__ __forceinline__ void init(int tid) {
         constexpr int CH = HD / 8;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
@@ -227,43 +222,22 @@ struct SlabLane {
             r[i] = pos / CH;
             c8[i] = 8 * ((pos % CH) ^ swz<HD>(r[i]));
             pos8[i] = pos * 8;
-            wbase[i] = (uint32_t)((pos & ~63) * 16);
             on[i] = pos < Slab<HD>::chunks;
         }
     }
 };
 
 // Copy stage rows row0 .. row0+31 of one [L][D] head slice into a slab (swizzled), zero-filled
-// beyond L and beyond D.  DMA = true: asynchronous LDS-DMA (needs `vec` inputs); the caller retires
-// it with wait_stages + barrier; exactly Slab<HD>::per_thread LDS-DMA instructions are issued by
-// every wave: a wave none of whose lanes has a row below L, or whose threads lie beyond a slab
-// smaller than the workgroup, issues a 4-byte placeholder copy into the sink instead, so that the
-// vmcnt arithmetic of wait_stages stays exact.  DMA = false: synchronous copy through registers
-// (any alignment).
-template <int HD, bool DMA>
+// beyond L and beyond D: a synchronous copy through registers that works for any alignment (`vec`
+// selects 16-byte loads when the rows allow them).
+template <int HD>
 __device__ __forceinline__ void fill_slab(const SlabLane<HD>& ln, elem_t* slab, const elem_t* g,
                                           int64_t sl, int row0, int L, int D, bool vec) {
-    const bool ragged = row0 + kStageRows > L;  // uniform
 #pragma unroll
     for (int i = 0; i < SlabLane<HD>::N; ++i) {
-        if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) {  // wave-uniform: a wave beyond the slab
-            if constexpr (DMA) dma4(g, ln.sink);
-            break;
-        }
+        if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) break;
         const int row = row0 + ln.r[i];
-        const bool valid = (row < L) && (ln.c8[i] < D);
-        if constexpr (DMA) {
-            // every lane of the wave writes base + 16*lane
-            if (valid) {
-                dma16(g + (int64_t)row * sl + ln.c8[i], lds_addr(slab) + ln.wbase[i]);
-            } else {
-                *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) = u32x4{0u, 0u, 0u, 0u};
-            }
-            if (ragged && __builtin_amdgcn_ballot_w64(valid) == 0) dma4(g, ln.sink);
-        } else {
-            *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) =
-                load8(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
-        }
+        *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) = load8(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
     }
 }
 
@@ -315,13 +289,6 @@ __device__ __forceinline__ void store_acc(elem_t* row, int d0, int hf, int D, co
                      T::pack2(acc[4 * jj + 2] * mul, acc[4 * jj + 3] * mul)};
         store4(row, d0 + 8 * jj + 4 * hf, D, val, vec);
     }
-}
-
-// Ring schedule shared by the streaming kernels: stages 0..n-1, R slots, stage s lives in slot
-// s % R.  Before consuming stage i the kernel has issued stages 0 .. issued_before(i)-1.
-__device__ __forceinline__ int ring_issued_before(int i, int R, int n) {
-    const int upto = (i == 0) ? R : i - 1 + R;
-    return upto < n ? upto : n;
 }
 
 }  // namespace sjvp

@@ -1,17 +1,17 @@
-// Fused attention-JVP forward kernel (gfx950).
+// Fused attention-JVP forward kernel, 32-wide form for inputs of any alignment (gfx950).
 //
 // Computes what semicat/jvp_utils/ryu_triton.py:73-291 computes - O, TO, M (= lse), MU, LI in one
 // online-softmax pass - with a different decomposition: a workgroup of four wavefronts owns 128
 // query rows of one (batch, head); each wavefront owns 32 of them as MFMA columns and walks over
-// the keys in stages of 32 streamed through an LDS ring (K, V, K_dot, V_dot; shared by the four
-// waves).  Scores are produced transposed (S^T = K Q^T) so that the running maximum, the exp-sum
-// and mu are per-lane scalars and the probability tile is directly the B operand of
-// O^T += V^T P^T.
+// the keys in stages of 32 copied through registers into one LDS stage (K, V, K_dot, V_dot; shared
+// by the four waves).  Scores are produced transposed (S^T = K Q^T) so that the running maximum,
+// the exp-sum and mu are per-lane scalars and the probability tile is directly the B operand of
+// O^T += V^T P^T.  Inputs whose rows are 16-byte aligned take the 16-wide kernel of sjvp_fwd16.hpp
+// instead; this one serves the rest (odd head dimensions, misaligned pointers or strides).
 #pragma once
 #include <type_traits>
 
 #include "sjvp_device.hpp"
-#include "sjvp_stream.hpp"
 
 namespace sjvp {
 
@@ -27,17 +27,12 @@ struct FwdParams {
     int vec;  // all tensors 16-byte aligned, strides % 8 == 0, D % 8 == 0
 };
 
-// LDS layout: [own: Q (and Q_dot) rows of the workgroup, one slab per wave - LDS-DMA path only]
-//             [ring: R slots of K, V (, K_dot, V_dot) stage slabs]
-// After the last stage the ring memory doubles as the per-wave staging tiles of the output stores.
-template <int HD, int R, bool JVP, bool DMA>
+// LDS layout: one stage of K, V (, K_dot, V_dot) slabs.
+template <int HD, bool JVP>
 struct FwdSmem {
-    static constexpr int nt = JVP ? 4 : 2;                      // tensors per stage
-    static constexpr int slot = nt * Slab<HD>::elems;            // elements per ring slot
-    static constexpr int own = DMA ? (JVP ? 2 : 1) * kWaves * Slab<HD>::elems : 0;
-    static constexpr int sink = (own + R * slot) * (int)sizeof(elem_t);
-    static constexpr int bytes = sink + kSinkBytes;
-    static_assert(!DMA || R * slot >= kWaves * StoreStage<HD>::elems, "ring too small to stage stores");
+    static constexpr int nt = JVP ? 4 : 2;             // tensors per stage
+    static constexpr int slot = nt * Slab<HD>::elems;  // elements of the stage
+    static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
 // The reference maximum of the online softmax is only raised when a new tile exceeds it by more
@@ -46,16 +41,13 @@ struct FwdSmem {
 // by the exp-sum is unaffected.  This keeps the accumulator rescale out of almost every tile.
 constexpr float kMaxSlack = 6.0f;
 
-template <typename T, int HD, int R, bool JVP, bool DMA>
+template <typename T, int HD, bool JVP>
 __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = FwdSmem<HD, R, JVP, DMA>;
-    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
-    elem_t* ring = own + SM::own;
+    elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
 
     constexpr int KC = HD / 16;  // k-chunks of the score contraction
     constexpr int DT = HD / 32;  // 32-wide tiles of the head dimension
-    constexpr int SPT = SM::nt * Slab<HD>::per_thread;  // LDS-DMA instructions per thread per stage
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -68,26 +60,14 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     const int b = bh / p.H, h = bh % p.H;
     const bool vec = p.vec != 0;
     SlabLane<HD> ln;
-    ln.init(tid, smem_raw + SM::sink);
+    ln.init(tid);
     const int qrow = qb * kOwned + wave * 32 + x;  // the query this lane owns
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
 
-    // Owned-side operands (B of S^T = K Q^T), kept in registers for the whole pass.  On the LDS-DMA
-    // path they are copied coalesced into LDS first (issued here, read after the first stages have
-    // been issued); otherwise every lane loads its own row.
+    // Owned-side operands (B of S^T = K Q^T), kept in registers for the whole pass.
     u32x4 qB[KC], tqB[KC];
-    if constexpr (DMA) {
-        const int r0 = qb * kOwned;
-#pragma unroll
-        for (int s4 = 0; s4 < kWaves; ++s4) {
-            fill_slab<HD, true>(ln, own + s4 * Slab<HD>::elems, p.q.head(b, h), p.q.sl, r0 + 32 * s4, p.Lq,
-                                p.D, true);
-            if constexpr (JVP)
-                fill_slab<HD, true>(ln, own + (kWaves + s4) * Slab<HD>::elems, p.tq.head(b, h), p.tq.sl,
-                                    r0 + 32 * s4, p.Lq, p.D, true);
-        }
-    } else {
+    {
         const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
 #pragma unroll
         for (int c = 0; c < KC; ++c) qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
@@ -102,14 +82,13 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     const elem_t* tkg = JVP ? p.tk.head(b, h) : nullptr;
     const elem_t* tvg = JVP ? p.tv.head(b, h) : nullptr;
 
-    auto issue = [&](int stage) {
-        elem_t* slot = ring + (stage % R) * SM::slot;
-        const int row0 = stage * kStageRows;
-        fill_slab<HD, DMA>(ln, slot, kg, p.k.sl, row0, p.Lk, p.D, vec);
-        fill_slab<HD, DMA>(ln, slot + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
+    auto fill = [&](int st) {
+        const int row0 = st * kStageRows;
+        fill_slab<HD>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (JVP) {
-            fill_slab<HD, DMA>(ln, slot + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
-            fill_slab<HD, DMA>(ln, slot + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -128,14 +107,11 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
         if constexpr (JVP) tacc[t] = f32x16{0};
     }
 
-    // One online-softmax step over NS consecutive stages (slots slot0, slot1): the score tiles of
-    // all NS stages are formed first, so that their MFMA chains, the exponentials and the output
-    // contractions of different stages overlap inside the wave.  Only the last stage of the step
-    // can be ragged.
-    auto compute = [&](const elem_t* slot0, const elem_t* slot1, int k0, auto ns_tag, auto ragged_tag) {
-        constexpr int NS = decltype(ns_tag)::value;
+    // One online-softmax step over the stage in LDS (keys k0 .. k0+31).
+    auto compute = [&](int k0, auto ragged_tag) {
+        constexpr int NS = 1;
         constexpr bool RAGGED = decltype(ragged_tag)::value;
-        const elem_t* slots[2] = {slot0, slot1};
+        const elem_t* slots[1] = {stage};
         f32x16 s[NS], ts[NS];
 #pragma unroll
         for (int g = 0; g < NS; ++g) {
@@ -223,60 +199,15 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     };
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
-    if constexpr (DMA) {
-        int issued = 0;
-        for (int s = 0; s < R && s < n; ++s, ++issued) issue(s);
-        // the owned rows were issued before these stages: they have landed once at most the
-        // stages' copies are outstanding
-        wait_stages<SPT>(issued);
+    for (int i = 0; i < n; ++i) {
+        __syncthreads();  // the previous stage is fully consumed
+        fill(i);
         __syncthreads();
-        read_b_operands<HD>(qB, own + wave * Slab<HD>::elems, x, hf);
-        if constexpr (JVP) read_b_operands<HD>(tqB, own + (kWaves + wave) * Slab<HD>::elems, x, hf);
+        if (!wave_active) continue;
+        const int k0 = i * kStageRows;
+        if (k0 + kStageRows > p.Lk) compute(k0, std::true_type{});
+        else compute(k0, std::false_type{});
     }
-    using one_t = std::integral_constant<int, 1>;
-    using two_t = std::integral_constant<int, 2>;
-    if constexpr (DMA && R >= 3) {
-        // two stages per step: stage i+1 must have landed as well, and the slot of stage i-1 (and
-        // i-2) is refilled afterwards
-        int next = (R < n) ? R : n;  // next stage to issue
-        for (int i = 0, last = 0; i < n; i = last + 1) {
-            // pair up with stage i+1 only if it has been issued already
-            last = (i + 1 < next) ? i + 1 : i;
-            wait_stages<SPT>(next - 1 - last);
-            __syncthreads();  // stages i..last have landed for every wave; stages < i are consumed
-            while (next < n && next < i + R) issue(next++);
-            if (!wave_active) continue;
-            const elem_t* s0 = ring + (i % R) * SM::slot;
-            const elem_t* s1 = ring + (last % R) * SM::slot;
-            const int k0 = i * kStageRows;
-            const bool ragged = (last + 1) * kStageRows > p.Lk;
-            if (last == i) {
-                if (ragged) compute(s0, s0, k0, one_t{}, std::true_type{});
-                else compute(s0, s0, k0, one_t{}, std::false_type{});
-            } else {
-                if (ragged) compute(s0, s1, k0, two_t{}, std::true_type{});
-                else compute(s0, s1, k0, two_t{}, std::false_type{});
-            }
-        }
-    } else {
-        for (int i = 0; i < n; ++i) {
-            if constexpr (DMA) {
-                wait_stages<SPT>(ring_issued_before(i, R, n) - 1 - i);
-                __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
-                if (i >= 1 && i - 1 + R < n) issue(i - 1 + R);
-            } else {
-                __syncthreads();
-                issue(i);
-                __syncthreads();
-            }
-            if (!wave_active) continue;
-            const elem_t* slot = ring + (i % R) * SM::slot;
-            const int k0 = i * kStageRows;
-            if (k0 + kStageRows > p.Lk) compute(slot, slot, k0, one_t{}, std::true_type{});
-            else compute(slot, slot, k0, one_t{}, std::false_type{});
-        }
-    }
-    if constexpr (DMA) __syncthreads();  // every wave is done reading the ring
     if (!wave_active) {
         // All 32 rows of this wave lie beyond Lq: their statistic rows get the values a zero
         // query row produces (and the reference initialises them with): log(Lk), 0, Lk.
@@ -313,25 +244,14 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
 #pragma unroll
             for (int j = 0; j < 16; ++j) tacc[d][j] -= cmu * acc[d][j];
     }
-    if constexpr (DMA) {
-        // every wave of the workgroup reaches this point (inactive ones returned above only after
-        // the loop): the ring is free and becomes the staging area of coalesced row stores
-        elem_t* stage_tile = ring + wave * StoreStage<HD>::elems;
-        const int row0 = qb * kOwned + wave * 32;
-        store_tile_coalesced<T, HD>(stage_tile, p.o.head(b, h), p.o.sl, row0, p.Lq, p.D, acc, inv_l, lane);
-        if constexpr (JVP)
-            store_tile_coalesced<T, HD>(stage_tile, p.to.head(b, h), p.to.sl, row0, p.Lq, p.D, tacc,
-                                        inv_l, lane);
-    } else {
-        if (!qvalid) return;
-        elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
+    if (!qvalid) return;
+    elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
-        if constexpr (JVP) {
-            elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
+    for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
+    if constexpr (JVP) {
+        elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
 #pragma unroll
-            for (int d = 0; d < DT; ++d) store_acc<T>(trow, 32 * d, hf, p.D, tacc[d], inv_l, vec);
-        }
+        for (int d = 0; d < DT; ++d) store_acc<T>(trow, 32 * d, hf, p.D, tacc[d], inv_l, vec);
     }
 }
 
