@@ -88,12 +88,14 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
              const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
 
 /*
- * The backward is two kernel launches: the row-owned one (dq, dtq, and the row sums it leaves in
- * the workspace) and the column-owned one (dk, dv, dtk, dtv), which consumes that workspace.
- * sjvp_bwd_parts() launches the selected ones with sjvp_bwd()'s arguments; sjvp_bwd() is
- * sjvp_bwd_parts(SJVP_BWD_ALL, ...).  It has no counterpart in the reference: it exists so that a
- * profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only valid on a
- * workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.
+ * sjvp_bwd() picks its launches by shape: for Lk <= 128 and D <= 64 (rows 16-byte aligned) one
+ * launch produces all six gradients and leaves the workspace untouched; otherwise the backward is
+ * a row-owned launch (dq, dtq, and the row sums it leaves in the workspace) followed by a
+ * column-owned one (dk, dv, dtk, dtv; two launches at D > 64), which consumes that workspace.
+ * sjvp_bwd_parts() runs the selected launches of that pair with sjvp_bwd()'s arguments;
+ * sjvp_bwd_parts(SJVP_BWD_ALL, ...) is sjvp_bwd().  It has no counterpart in the reference: it exists
+ * so that a profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only
+ * valid on a workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.
  */
 enum sjvp_bwd_part { SJVP_BWD_ROW = 1, SJVP_BWD_COL = 2, SJVP_BWD_ALL = 3 };
 int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const void* tq,

@@ -19,10 +19,6 @@
 
 namespace sjvp {
 
-#ifndef SJVP_SCHED_BARRIER
-#define SJVP_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0)
-#endif
-
 // LDS layout: [own K, K_dot: four slabs each][own V, V_dot: four slabs each; once they have been
 // read into registers the same memory is the bounce tile dS (, dS_dot): [128 keys][32 queries + pad]]
 // [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d][sink]
@@ -230,10 +226,10 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         };
         // the second tile's MFMA chains run under the first tile's pointwise arithmetic
         scores(0);
-        SJVP_SCHED_BARRIER;
+        __builtin_amdgcn_sched_barrier(0);
         scores(1);
         pointwise(0);
-        SJVP_SCHED_BARRIER;
+        __builtin_amdgcn_sched_barrier(0);
         // the first transposed operands of the output contractions are fetched under the second
         // tile's pointwise arithmetic
         const u32x4 aq0 = lds_a_tr16<HD>(sQ, 0, lane);
@@ -243,7 +239,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             ag0 = lds_a_tr16<HD>(sG, 0, lane);
         }
         if constexpr (HAS_DO) ado0 = lds_a_tr16<HD>(sDO, 0, lane);
-        SJVP_SCHED_BARRIER;
+        __builtin_amdgcn_sched_barrier(0);
         pointwise(1);
         const u32x4 pB = pack_b16<T>(s[0], s[1]);
         const u32x4 dsB = pack_b16<T>(xy[0], xy[1]);
