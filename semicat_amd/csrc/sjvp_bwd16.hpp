@@ -112,7 +112,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
         ++issued;
     };
-    while (issued < R && issued < ns) issue_next();
+    issue_next();
     const float sl2 = p.scale * kLog2e;
 
     // Row sums of a landed stage: thread t < 256 handles row t/8, columns 8*(t%8) .. +7; the eight
@@ -341,8 +341,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
     };
 
-    wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
+    // Only the own rows and stage 0 are waited for here; the later stages are issued once these
+    // have landed, so that their copies run under the arithmetic instead of ahead of it.
+    wait_stages<SPT>(0);
     __syncthreads();
+    if (issued < ns) issue_next();
     {
         const int r = 16 * (wave & 1) + n;
         const int sidx = wave >> 1;
@@ -358,15 +361,15 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
         __syncthreads();
-            if (i >= 1 && issued < ns) issue_next();
+        if (issued < ns && issued < i + R) issue_next();  // into the slot of stage issued - R <= i - 1
         elem_t* slot = ring + (i % R) * SM::slot;
-            if (wave_active) tile(slot);
-            if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
+        if (wave_active) tile(slot);
+        if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
         __syncthreads();
-            if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
-            if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
+        if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
+        if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
         else row_outputs(i * kStageRows, std::false_type{});
-        }
+    }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
