@@ -110,6 +110,8 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=
     lse = _stat(lse, "M", B, H, Lr, dev)
     mu = _stat(mu, "MU", B, H, Lr, dev)
     li = _stat(li, "LI", B, H, Lr, dev) if (with_li or li is not None) else None
+    if B * H * Lq == 0 and not _plan:  # nothing to compute (an empty batch slice): no launch
+        return o, to, lse, mu, li
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
@@ -139,6 +141,8 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
         o = torch.empty((B, H, Lq, D), device=dev, dtype=dt)
     _check_bhld("y", o, (B, H, Lq, D), dt, dev)
     lse = _stat(lse, "M", B, H, stat_rows(Lq), dev)
+    if B * H * Lq == 0:
+        return o, lse
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
@@ -208,6 +212,8 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         _check_bhld("dtv", dtv, (B, H, Lk, D), dt, dev)
     else:
         dtq = dtk = dtv = None
+    if B * H * Lq == 0 and not _plan:
+        return dq, dk, dv, dtq, dtk, dtv
     lib = _lib.load()
     nbytes = lib.sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype_tag)
     if workspace is None:

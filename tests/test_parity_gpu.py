@@ -290,3 +290,16 @@ def test_planned_launches_match_direct_calls(K):
     torch.cuda.synchronize()
     for a, b in zip((o, to, lse, mu) + tuple(g), (o2, to2, lse2, mu2) + tuple(g2)):
         assert torch.equal(a, b)
+
+
+def test_empty_batch_returns_empty_results(K):
+    """A batch slice of zero samples (the cross-entropy share of a step whose whole batch takes the
+    self-distillation loss, semicat.py:186-187) yields empty outputs without a launch."""
+    z = lambda *shape: torch.empty(shape, device="cuda", dtype=torch.bfloat16)
+    q = z(0, 3, 128, 64)
+    o, lse = K.attention_forward(q, q, q)
+    assert o.shape == (0, 3, 128, 64) and lse.shape == (0, 3, 128)
+    o, to, lse, mu, li = K.attention_jvp_forward(q, q, q, q, q, q)
+    assert o.shape == to.shape == (0, 3, 128, 64)
+    grads = K.attention_jvp_backward(q, q, q, q, q, q, o, to, lse, mu, dO=q, dTO=q)
+    assert all(g.shape == (0, 3, 128, 64) for g in grads)
