@@ -73,6 +73,9 @@ struct Ring {
     static constexpr int pair = HD == 128 ? 2 : 3;     // row-owned / column-owned backward pair
 };
 
+// key-axis length from which the forward takes two stages per barrier
+constexpr int kFwdPairedFrom = 256;
+
 // 32-wide forward for inputs of any alignment (register-staged copies, one stage in LDS)
 template <typename T, int HD>
 int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
@@ -87,6 +90,14 @@ int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     constexpr int R = Ring<HD>::fwd16;
     constexpr int RP = Ring<HD>::fwd16_primal;
     constexpr int OCC = HD == 128 ? 2 : 4;
+    if (p.Lk >= kFwdPairedFrom) {
+        // long key axes: two stages per barrier over a ring of four slots in the same LDS footprint
+        if (jvp)
+            return launch(fwd16_kernel<T, HD, 4, true, OCC, 2>, grid, Fwd16Smem<HD, 4, true, 2>::bytes, stream,
+                          p, kThreads16);
+        return launch(fwd16_kernel<T, HD, 4, false, OCC, 2>, grid, Fwd16Smem<HD, 4, false, 2>::bytes, stream,
+                      p, kThreads16);
+    }
     if (jvp)
         return launch(fwd16_kernel<T, HD, R, true, OCC>, grid, Fwd16Smem<HD, R, true>::bytes, stream, p,
                       kThreads16);

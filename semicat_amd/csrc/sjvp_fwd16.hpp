@@ -12,25 +12,31 @@
 
 namespace sjvp {
 
-// LDS layout: [own: Q (, Q_dot) rows of the workgroup, four slabs each][ring: R slots of K, V
-// (, K_dot, V_dot) stage slabs][sink].  After the last stage the ring doubles as the per-wave
-// staging tiles of the output stores.
-template <int HD, int R, bool JVP>
+// LDS layout, SPB = 1 (one stage per barrier): [own: Q (, Q_dot) rows of the workgroup, four slabs
+// each][ring: R slots of K, V (, K_dot, V_dot) stage slabs][sink].  SPB = 2 (long key axes: two stages
+// per barrier, half as many barriers): [ring of four slots][sink]; the own rows, which every wave
+// moves into registers before the first stage is consumed, land in slots 2 and 3 (exactly their
+// size), which then join the ring.  After the last stage the ring doubles as the per-wave staging
+// tiles of the output stores.
+template <int HD, int R, bool JVP, int SPB = 1>
 struct Fwd16Smem {
     static constexpr int nt = JVP ? 4 : 2;
     static constexpr int slot = nt * Slab<HD>::elems;
     static constexpr int own = (JVP ? 2 : 1) * 4 * Slab<HD>::elems;
-    static constexpr int sink = (own + R * slot) * (int)sizeof(elem_t);
+    static_assert(SPB == 1 || (SPB == 2 && R == 4 && own == 2 * slot), "SPB = 2 needs a ring of four slots");
+    static constexpr int own_off = SPB == 2 ? 2 * slot : 0;
+    static constexpr int ring_off = SPB == 2 ? 0 : own;
+    static constexpr int sink = (SPB == 2 ? R * slot : own + R * slot) * (int)sizeof(elem_t);
     static constexpr int bytes = sink + kSink16;
     static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool JVP, int OCC>
+template <typename T, int HD, int R, bool JVP, int OCC, int SPB = 1>
 __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    using SM = Fwd16Smem<HD, R, JVP>;
-    elem_t* own = reinterpret_cast<elem_t*>(smem_raw);
-    elem_t* ring = own + SM::own;
+    using SM = Fwd16Smem<HD, R, JVP, SPB>;
+    elem_t* own = reinterpret_cast<elem_t*>(smem_raw) + SM::own_off;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw) + SM::ring_off;
     constexpr int SE = Slab<HD>::elems;
     constexpr int KC = HD / 32;  // k-chunks of the score contraction
     constexpr int DT = HD / 16;  // 16-wide tiles of the head dimension
@@ -72,7 +78,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows);
         ++issued;
     };
-    while (issued < R && issued < ns) issue_next();
+    while (issued < (SPB == 2 ? 2 : R) && issued < ns) issue_next();
 
     const float sl2 = p.scale * kLog2e;
     float m_i = -INFINITY;     // reference maximum (same in the four lanes of a query)
@@ -88,13 +94,20 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         tacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    wait_stages<SPT>(issued - 1);  // the own rows and stage 0 were issued before the other stages
+    // SPB = 1: the own rows and stage 0 were issued before the other stages; SPB = 2: everything
+    wait_stages<SPT>(SPB == 2 ? 0 : issued - 1);
     __syncthreads();
     u32x4 qB[KC], tqB[KC];
     {
         const int r = 16 * (wave & 1) + n;
         read_b_operands16<HD>(qB, own + (wave >> 1) * SE, r, g);
         if constexpr (JVP) read_b_operands16<HD>(tqB, own + (4 + (wave >> 1)) * SE, r, g);
+    }
+    if constexpr (SPB == 2) {
+        // the operands must have arrived in registers before the copies below overwrite their slots
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        while (issued < R && issued < ns) issue_next();
     }
 
     auto compute = [&](const elem_t* slot, int k0) {
@@ -170,17 +183,20 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         }
     };
 
-    for (int i = 0; i < ns; ++i) {
+    for (int i = 0; i < ns; i += SPB) {
         if (i > 0) {
-            wait_stages<SPT>(issued - 1 - i);
-            __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
-            if (issued < ns) issue_next();
+            // the stages of this step have landed for every wave; those of the last step are consumed
+            wait_stages<SPT>(SPB == 2 ? 0 : issued - 1 - i);
+            __syncthreads();
+#pragma unroll
+            for (int u = 0; u < SPB; ++u)
+                if (issued < ns) issue_next();
         }
         if (!wave_active) continue;
-        const elem_t* slot = ring + (i % R) * SM::slot;
-        const int k0 = i * kStageRows;
-        compute(slot, k0);
-        }
+#pragma unroll
+        for (int u = 0; u < SPB; ++u)
+            if (i + u < ns) compute(ring + ((i + u) % R) * SM::slot, (i + u) * kStageRows);
+    }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
     const int64_t so = (int64_t)bh * p.Lr + qrow;
     if (!wave_active) {
