@@ -132,21 +132,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             if constexpr (HAS_DO) d4 = *reinterpret_cast<const u32x4*>(slot + oDO + off);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float o0 = T::to_float((elem_t)(o4[i] & 0xffffu));
-                const float o1 = T::to_float((elem_t)(o4[i] >> 16));
                 if constexpr (HAS_G) {
-                    const float g0 = T::to_float((elem_t)(g4[i] & 0xffffu));
-                    const float g1 = T::to_float((elem_t)(g4[i] >> 16));
-                    const float t0 = T::to_float((elem_t)(t4[i] & 0xffffu));
-                    const float t1 = T::to_float((elem_t)(t4[i] >> 16));
-                    s4 += g0 * o0 + g1 * o1;
-                    s7d += g0 * t0 + g1 * t1;
+                    s4 = T::dot2(g4[i], o4[i], s4);
+                    s7d = T::dot2(g4[i], t4[i], s7d);
                 }
-                if constexpr (HAS_DO) {
-                    const float d0 = T::to_float((elem_t)(d4[i] & 0xffffu));
-                    const float d1 = T::to_float((elem_t)(d4[i] >> 16));
-                    s7d += d0 * o0 + d1 * o1;
-                }
+                if constexpr (HAS_DO) s7d = T::dot2(d4[i], o4[i], s7d);
             }
         }
         s4 = sum8(s4);

@@ -30,10 +30,7 @@ template <typename T>
 __device__ __forceinline__ float dot8(const u32x4& a, const u32x4& b) {
     float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        s += T::to_float((elem_t)(a[i] & 0xffffu)) * T::to_float((elem_t)(b[i] & 0xffffu));
-        s += T::to_float((elem_t)(a[i] >> 16)) * T::to_float((elem_t)(b[i] >> 16));
-    }
+    for (int i = 0; i < 4; ++i) s = T::dot2(a[i], b[i], s);
     return s;
 }
 

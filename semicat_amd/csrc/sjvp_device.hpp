@@ -68,6 +68,11 @@ struct Bf16 {
     static __device__ __forceinline__ float to_float(elem_t x) {
         return __builtin_bit_cast(float, (uint32_t)x << 16);
     }
+    // a.lo * b.lo + a.hi * b.hi + c on a packed pair, accumulated in fp32 (v_dot2c_f32_bf16)
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c,
+                                               false);
+    }
 };
 
 struct Fp16 {
@@ -85,6 +90,9 @@ struct Fp16 {
     }
     static __device__ __forceinline__ float to_float(elem_t x) {
         return (float)__builtin_bit_cast(_Float16, x);
+    }
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
     }
 };
 
