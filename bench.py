@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention-JVP forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--graph] [--no-cpu-baseline] [--calib-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--graph] [--no-cpu-baseline] [--no-cold] [--calib-copy]
 
 A step is one pass of the hot path over one batch: the fused forward (O, TO, lse, mu) followed by
 the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
@@ -32,8 +32,8 @@ NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
 # kernel of --calib-copy: one FETCH_SIZE unit is 2 KiB, one WRITE_SIZE unit 1 KiB there).
 MEASURED_TRAFFIC_BYTES = {
-    "fwd16_kernel": (2 * 36934.6 + 25344.0) * 1024,
-    "bwd_fused16_kernel": (2 * 61940.6 + 73728.0) * 1024,
+    "fwd16_kernel": (2 * 36937.8 + 25344.0) * 1024,
+    "bwd_fused16_kernel": (2 * 61936.3 + 73728.0) * 1024,
 }
 
 
@@ -92,6 +92,7 @@ def main() -> int:
                     help="replay a HIP graph of one step instead of launching through the C ABI every step")
     ap.add_argument("--no-graph", action="store_true", help="(default behaviour; kept for old command lines)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache timing over rotating buffer sets")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device copy (reference point for rocprofv3 --pmc byte counters)")
     a = ap.parse_args()
@@ -152,21 +153,52 @@ def main() -> int:
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
 
-        # Per-kernel durations: HIP events on the launch stream around runs of one kernel launched
-        # alone (every kernel sees the same buffers as in the timed steps).
-        def timed(fn, n=100):
-            for _ in range(10):
-                fn()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(n):
-                fn()
-            e1.record(stream)
-            e1.synchronize()
-            return e0.elapsed_time(e1) / n  # ms
+        # Per-kernel durations: the same steps once more, now with HIP events on the launch stream
+        # around every launch (forward and backward alternate exactly as in the timed region, so
+        # each kernel meets the caches in the state the other one left them in).
+        n_ev = min(a.steps, 200)
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n_ev)]
+        for _ in range(3):
+            step()
+        for e in evs:
+            e[0].record(stream)
+            fwd()
+            e[1].record(stream)
+            bwd()
+            e[2].record(stream)
+        stream.synchronize()
+        fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / n_ev
+        bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / n_ev
 
-        fwd_ms = timed(fwd)
-        bwd_ms = timed(bwd)
+        # Cold caches: the same step over six independent sets of buffers (1.2 GB in all, several
+        # times the 256 MB Infinity Cache) used in rotation, so that no launch finds its operands
+        # in a cache; reported beside the headline figure, which re-uses one set as a training
+        # step does between a layer's forward and backward.
+        cold_ms = None
+        if not a.no_cold:
+            sets = []
+            for _ in range(6):
+                y = {n: torch.empty_like(x[n]).copy_(x[n]) for n in NAMES}
+                o2, to2 = torch.empty_like(q), torch.empty_like(q)
+                lse2, mu2 = torch.empty_like(lse), torch.empty_like(lse)
+                g2 = tuple(torch.empty_like(q) for _ in range(6))
+                f2, _ = kernels.plan_forward(*(y[n] for n in NAMES[:6]), o=o2, to=to2, lse=lse2, mu=mu2,
+                                             with_li=False)
+                b2, _ = kernels.plan_backward(*(y[n] for n in NAMES[:6]), o2, to2, lse2, mu2, dO=y["dO"],
+                                              dTO=y["dTO"], grads=g2, workspace=workspace)
+                sets.append((f2, b2, y, o2, to2, lse2, mu2, g2))
+            n_cold = 60
+            for i in range(12):
+                sets[i % 6][0]()
+                sets[i % 6][1]()
+            stream.synchronize()
+            t0 = time.perf_counter()
+            for i in range(n_cold):
+                sets[i % 6][0]()
+                sets[i % 6][1]()
+            stream.synchronize()
+            cold_ms = (time.perf_counter() - t0) / n_cold * 1e3
+            del sets
 
         if a.calib_copy:
             # a plain copy of known size, for scaling the FETCH_SIZE / WRITE_SIZE hardware counters
@@ -231,6 +263,8 @@ def main() -> int:
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
+        "cold_ms_per_step": cold_ms,
+        "cold_tflops": None if cold_ms is None else step_flops() / (cold_ms * 1e-3) / 1e12,
         "kernels": {n: {"ms": w["ms"], "GBps": w["GBps"], "TFLOPs": w["TFLOPs"]} for n, w in work.items()},
         "roofline": roofline,
         "device": torch.cuda.get_device_name(0),
