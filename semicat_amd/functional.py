@@ -67,8 +67,9 @@ class SDPAJVPForwardFunction(torch.autograd.Function):
         # y and M (allocated by SDPAFunction.forward) are filled in place by the fused kernel.
         # LI, which the reference also keeps (functional.py:57-59), is not needed by the backward.
         with torch.no_grad():
-            _, t_y, _, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y, lse=M,
-                                                             with_li=False)
+            # the tangent output takes the memory layout of the primal output
+            _, t_y, _, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y,
+                                                             to=torch.empty_like(y), lse=M, with_li=False)
         return t_y, MU
 
     @staticmethod
@@ -86,24 +87,34 @@ class SDPAJVPForwardFunction(torch.autograd.Function):
         return *grads, None, None
 
 
+def _empty_output(q: Tensor, d_v: int, seq_major: bool) -> Tensor:
+    """A ``[B,H,S,D]`` output buffer: contiguous as the reference allocates it (functional.py:224-227),
+    or, for callers that work in ``[B,S,H,D]``, a view of a ``[B,S,H,D]``-contiguous buffer, so that
+    handing the result back in their layout needs no copy (the kernels write through strides)."""
+    B, H, S, _ = q.shape
+    if seq_major:
+        return torch.empty((B, S, H, d_v), device=q.device, dtype=q.dtype).transpose(1, 2)
+    return torch.empty((B, H, S, d_v), device=q.device, dtype=q.dtype)
+
+
 class SDPAFunction(torch.autograd.Function):
     """The op under forward-mode AD (functional.py:216-268)."""
 
     @staticmethod
-    def forward(q, k, v):
-        B, H, S, D = q.shape
-        y = torch.empty((B, H, S, v.shape[-1]), device=q.device, dtype=q.dtype)
-        M = torch.empty((B, H, kernels.stat_rows(S)), device=q.device, dtype=torch.float32)
+    def forward(q, k, v, seq_major=False):
+        y = _empty_output(q, v.shape[-1], seq_major)
+        M = torch.empty((q.shape[0], q.shape[1], kernels.stat_rows(q.shape[2])), device=q.device,
+                        dtype=torch.float32)
         return y, M
 
     @staticmethod
     def setup_context(ctx: Any, inputs: tuple[Any, ...], output: Any) -> Any:
-        ctx.save_for_forward(*inputs, *output)
-        ctx.save_for_backward(*inputs, *output)
+        ctx.save_for_forward(*inputs[:3], *output)
+        ctx.save_for_backward(*inputs[:3], *output)
         ctx.set_materialize_grads(False)
 
     @staticmethod
-    def jvp(ctx, t_q, t_k, t_v):
+    def jvp(ctx, t_q, t_k, t_v, *_):
         q, k, v, y, M = ctx.saved_for_forward
         t_q = torch.zeros_like(q) if t_q is None else t_q
         t_k = torch.zeros_like(k) if t_k is None else t_k
@@ -114,19 +125,19 @@ class SDPAFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_y, d_M):
         if d_y is None:
-            return None, None, None
+            return None, None, None, None
         q, k, v, y, M = ctx.saved_tensors
         with torch.no_grad():
             dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
-        return dq, dk, dv
+        return dq, dk, dv, None
 
 
 class SDPAPrimalFunction(torch.autograd.Function):
     """The op without forward-mode tangents: plain attention with the primal-only kernels."""
 
     @staticmethod
-    def forward(ctx, q, k, v):
-        y, M = kernels.attention_forward(q, k, v)
+    def forward(ctx, q, k, v, seq_major=False):
+        y, M = kernels.attention_forward(q, k, v, o=_empty_output(q, v.shape[-1], seq_major))
         ctx.save_for_backward(q, k, v, y, M)
         return y
 
@@ -134,7 +145,7 @@ class SDPAPrimalFunction(torch.autograd.Function):
     def backward(ctx, d_y):
         q, k, v, y, M = ctx.saved_tensors
         dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
-        return dq, dk, dv
+        return dq, dk, dv, None
 
 
 @torch._dynamo.disable
@@ -142,10 +153,15 @@ def sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
     """Fused scaled-dot-product attention with forward-mode (jvp) support; ``[B,H,S,D]`` bf16/fp16
     (functional.py:272-307).  Usage: ``y, t_y = torch.func.jvp(sdpa_jvp, (q, k, v), (t_q, t_k, t_v))``
     or wrap a whole model that calls it in ``torch.func.jvp``; both outputs support ``backward``."""
+    return _sdpa(q, k, v, seq_major=False)
+
+
+@torch._dynamo.disable
+def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool) -> Tensor:
     if _has_tangent(q) or _has_tangent(k) or _has_tangent(v):
-        y, _ = SDPAFunction.apply(q, k, v)
+        y, _ = SDPAFunction.apply(q, k, v, seq_major)
         return y
-    return SDPAPrimalFunction.apply(q, k, v)
+    return SDPAPrimalFunction.apply(q, k, v, seq_major)
 
 
 def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
@@ -156,7 +172,9 @@ def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
         q = q.to(torch.bfloat16)
         k = k.to(torch.bfloat16)
         v = v.to(torch.bfloat16)
-    y = sdpa_jvp(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2))
+    # The reference returns a [B,S,H,D] view of a [B,H,S,D]-contiguous result, which its callers then
+    # copy when they flatten the heads (duo.py:155); here the kernels write [B,S,H,D] memory directly.
+    y = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), seq_major=True).transpose(1, 2)
     if y.dtype != orig_dtype:
         y = y.to(orig_dtype)
-    return y.transpose(1, 2)
+    return y

@@ -119,6 +119,27 @@ def test_through_a_module_with_scalar_time_tangent(monkeypatch):
     assert lin.weight.grad.abs().sum() > 0
 
 
+def test_seq_major_results_need_no_copy(monkeypatch):
+    """safe_sdpa_jvp hands back [B,S,H,D]-contiguous results (primal and tangent, with and without
+    forward-mode AD), so flattening the heads as duo.py:155 does is a view; sdpa_jvp keeps the
+    reference's [B,H,S,D]-contiguous result (functional.py:224-227)."""
+    eager_backend.install(monkeypatch)
+    x = orc.make_inputs(2, 3, 12, 12, 16, seed=3, dtype=torch.bfloat16)
+    bshd = [x[n].transpose(1, 2).contiguous() for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(functional.safe_sdpa_jvp, tuple(bshd[:3]), tuple(bshd[3:]))
+    plain = functional.safe_sdpa_jvp(*bshd[:3])
+    for t in (y, ty, plain):
+        assert t.shape == (2, 12, 3, 16) and t.is_contiguous()
+        assert t.reshape(2, 12, 48).data_ptr() == t.data_ptr()
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    assert orc.rel_frobenius(y.transpose(1, 2), ref["O"]) < 3e-2
+    assert orc.rel_frobenius(ty.transpose(1, 2), ref["TO"]) < 3e-2
+    assert orc.rel_frobenius(plain.transpose(1, 2), ref["O"]) < 3e-2
+    y2, _ = torch.func.jvp(functional.sdpa_jvp, tuple(x[n] for n in orc.TENSOR_ORDER[:3]),
+                           tuple(x[n] for n in orc.TENSOR_ORDER[3:6]))
+    assert y2.is_contiguous() and y2.shape == (2, 3, 12, 16)
+
+
 def test_launchers_refuse_cpu_tensors():
     """No CPU fallback: the real launchers raise on non-GPU tensors."""
     q = torch.zeros(1, 1, 8, 16, dtype=torch.bfloat16)

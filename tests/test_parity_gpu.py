@@ -247,6 +247,16 @@ def test_autograd_end_to_end_on_gpu(K):
     y2 = safe_sdpa_jvp(q32, k32, v32)
     assert y2.dtype == torch.float32 and y2.shape == (B, L, H, D)
     assert orc.rel_frobenius(y2.transpose(1, 2).cpu(), ref["O"]) <= TOL_16BIT
+    # under forward-mode AD through the [B,S,H,D] wrapper: results land in [B,S,H,D] memory (no copy
+    # when the caller flattens the heads), gradients reach the [B,S,H,D] leaves
+    bshd = [x[n].cuda().transpose(1, 2).contiguous().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
+    y3, ty3 = torch.func.jvp(safe_sdpa_jvp, tuple(bshd[:3]), tuple(bshd[3:]))
+    assert y3.is_contiguous() and ty3.is_contiguous() and y3.shape == (B, L, H, D)
+    w_o, w_to = x["dO"].cuda().float().transpose(1, 2), x["dTO"].cuda().float().transpose(1, 2)
+    ((y3.float() * w_o).sum() + (ty3.float() * w_to).sum()).backward()
+    res3 = {"O": y3.detach().transpose(1, 2).cpu(), "TO": ty3.detach().transpose(1, 2).cpu(),
+            **{n: l.grad.transpose(1, 2).cpu() for n, l in zip(GRADS, bshd)}}
+    assert_parity(res3, ref, 1.2e-2, label="autograd, [B,S,H,D] caller")
 
 
 def test_reference_signature_wrappers(K):
