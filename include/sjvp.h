@@ -40,7 +40,7 @@ extern "C" {
 
 #define SJVP_VERSION 1
 
-enum sjvp_dtype { SJVP_BF16 = 0, SJVP_FP16 = 1 };
+enum sjvp_dtype { SJVP_BF16 = 0, SJVP_FP16 = 1, SJVP_FP32 = 2 /* sjvp_rope only */ };
 
 enum sjvp_status {
     SJVP_OK = 0,
@@ -51,7 +51,8 @@ enum sjvp_status {
     SJVP_ERR_WORKSPACE = -5, /* workspace NULL or smaller than sjvp_bwd_workspace_bytes()    */
     SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (hipGetLastError)           */
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
-    SJVP_ERR_PARTS = -8      /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
+    SJVP_ERR_PARTS = -8,     /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
+    SJVP_ERR_ROTARY = -9     /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16 */
 };
 
 /* Indices into the stride tables: strides[3*i + {0,1,2}] = (batch, head, sequence) strides in
@@ -109,6 +110,26 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
  * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,
  * flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
+
+/*
+ * Rotary position embedding of n (1..4) tensors of one shape in one launch, with the cast to
+ * out_dtype and any change of layout folded in.  For position l, i < rot_dim/2 and h = rot_dim/2:
+ *   y[b,h,l,i]     = x[b,h,l,i]   cos[l,i] - sign x[b,h,l,i+h] sin[l,i]
+ *   y[b,h,l,i+h]   = x[b,h,l,i+h] cos[l,i] + sign x[b,h,l,i]   sin[l,i]
+ * with sign = +1, or -1 when `inverse` is non-zero; columns from rot_dim on are copied.  This is the
+ * non-interleaved rotation that semicat/net/duo.py:45-55 applies to q and k before the attention op
+ * through flash_attn.layers.rotary.apply_rotary_emb_torch (flash_attn 2.8.3, not vendored by the
+ * reference), there as separate fp32 PyTorch operations.  The map is linear in x: the same call
+ * rotates forward-mode tangents, and the inverse rotation back-propagates cotangents.
+ *   x[i], y[i]   [B,H,L,D] views, unit last stride; strides[6*i + {0,1,2}] = (batch, head, sequence)
+ *                element strides of x[i], strides[6*i + {3,4,5}] those of y[i]; y[i] may alias x[i]
+ *                only if both have the same dtype and strides
+ *   cos, sin     fp32 [L][rot_dim/2] with row stride cs_stride (elements)
+ *   in_dtype, out_dtype   SJVP_BF16, SJVP_FP16 or SJVP_FP32 (not bf16 on one side and fp16 on the other)
+ */
+int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides /* [n*6] */,
+              const float* cos, const float* sin, int64_t cs_stride, int B, int H, int L, int D,
+              int rot_dim, int in_dtype, int out_dtype, int inverse, void* stream);
 
 /* Static, NUL-terminated description of a status code. */
 const char* sjvp_strerror(int status);

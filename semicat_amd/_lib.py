@@ -10,6 +10,7 @@ from . import build as _build
 
 SJVP_BF16 = 0
 SJVP_FP16 = 1
+SJVP_FP32 = 2  # sjvp_rope only
 
 SJVP_OK = 0
 SJVP_ERR_NULL = -1
@@ -20,6 +21,7 @@ SJVP_ERR_WORKSPACE = -5
 SJVP_ERR_LAUNCH = -6
 SJVP_ERR_COTANGENT = -7
 SJVP_ERR_PARTS = -8
+SJVP_ERR_ROTARY = -9
 
 SJVP_BWD_ROW = 1
 SJVP_BWD_COL = 2
@@ -29,8 +31,8 @@ F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
 B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
-EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_workspace_bytes", "sjvp_strerror",
-           "sjvp_version")
+EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_workspace_bytes", "sjvp_rope",
+           "sjvp_strerror", "sjvp_version")
 
 _lock = threading.Lock()
 _lib = None
@@ -64,6 +66,9 @@ def load() -> ctypes.CDLL:
             lib.sjvp_bwd_parts.restype = i
             lib.sjvp_bwd_workspace_bytes.argtypes = [i] * 6
             lib.sjvp_bwd_workspace_bytes.restype = ctypes.c_size_t
+            vpp = ctypes.POINTER(ctypes.c_void_p)
+            lib.sjvp_rope.argtypes = [i, vpp, vpp, i64p, vp, vp, ctypes.c_int64] + [i] * 8 + [vp]
+            lib.sjvp_rope.restype = i
             lib.sjvp_strerror.argtypes = [i]
             lib.sjvp_strerror.restype = ctypes.c_char_p
             lib.sjvp_version.argtypes = []

@@ -10,6 +10,7 @@
 #include "sjvp_bwd16x.hpp"
 #include "sjvp_fwd.hpp"
 #include "sjvp_fwd16.hpp"
+#include "sjvp_rope.hpp"
 
 using namespace sjvp;
 
@@ -311,6 +312,64 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
                               : bwd_dtype<Fp16>(p, B * H, has_do, has_g, parts, s);
 }
 
+int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides, const float* cos,
+              const float* sin, int64_t cs_stride, int B, int H, int L, int D, int rot_dim, int in_dtype,
+              int out_dtype, int inverse, void* stream) {
+    if (!x || !y || !strides || !cos || !sin) return SJVP_ERR_NULL;
+    if (n < 1 || n > kRopeMaxTensors) return SJVP_ERR_ROTARY;
+    if (B < 1 || H < 1 || L < 1 || D < 1) return SJVP_ERR_SHAPE;
+    if (rot_dim < 2 || rot_dim > D || (rot_dim & 1)) return SJVP_ERR_ROTARY;
+    auto known = [](int d) { return d == SJVP_BF16 || d == SJVP_FP16 || d == SJVP_FP32; };
+    if (!known(in_dtype) || !known(out_dtype)) return SJVP_ERR_DTYPE;
+    if (in_dtype != SJVP_FP32 && out_dtype != SJVP_FP32 && in_dtype != out_dtype) return SJVP_ERR_ROTARY;
+    const int half = rot_dim / 2;
+    const int in_bytes = in_dtype == SJVP_FP32 ? 4 : 2, out_bytes = out_dtype == SJVP_FP32 ? 4 : 2;
+
+    RopeParams p;
+    // eight columns per thread need every row start and the second half of a pair 16-byte aligned
+    bool vec = half % 8 == 0 && (D - rot_dim) % 8 == 0 && aligned16(cos) && aligned16(sin) && cs_stride % 4 == 0;
+    for (int i = 0; i < kRopeMaxTensors; ++i) {
+        const int j = i < n ? i : 0;  // unused slots repeat tensor 0 (never dereferenced: grid.y = n)
+        if (!x[j] || !y[j]) return SJVP_ERR_NULL;
+        p.x[i] = x[j];
+        p.y[i] = y[j];
+        for (int d = 0; d < 3; ++d) {
+            p.xs[i][d] = strides[6 * j + d];
+            p.ys[i][d] = strides[6 * j + 3 + d];
+            vec = vec && (p.xs[i][d] * in_bytes) % 16 == 0 && (p.ys[i][d] * out_bytes) % 16 == 0;
+        }
+        vec = vec && aligned16(x[j]) && aligned16(y[j]);
+    }
+    p.cos = cos;
+    p.sin = sin;
+    p.cs = cs_stride;
+    p.H = H;
+    p.L = L;
+    p.D = D;
+    p.half = half;
+    const int w = vec ? 8 : 1;
+    p.units = half / w + (D - rot_dim) / w;
+    p.total = (int64_t)B * H * L * p.units;
+    p.sign = inverse ? -1.0f : 1.0f;
+    const int64_t blocks = (p.total + kRopeThreads - 1) / kRopeThreads;
+    if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
+
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)n), dim3(kRopeThreads), 0,
+                           static_cast<hipStream_t>(stream), p);
+        return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
+    };
+    auto by_out = [&](auto in_tag) {
+        using IN = decltype(in_tag);
+        if (out_dtype == SJVP_FP32) return vec ? go(rope_kernel<IN, F32, true>) : go(rope_kernel<IN, F32, false>);
+        if (out_dtype == SJVP_BF16) return vec ? go(rope_kernel<IN, Bf16, true>) : go(rope_kernel<IN, Bf16, false>);
+        return vec ? go(rope_kernel<IN, Fp16, true>) : go(rope_kernel<IN, Fp16, false>);
+    };
+    if (in_dtype == SJVP_FP32) return by_out(F32{});
+    if (in_dtype == SJVP_BF16) return by_out(Bf16{});
+    return by_out(Fp16{});
+}
+
 const char* sjvp_strerror(int status) {
     switch (status) {
         case SJVP_OK: return "ok";
@@ -322,6 +381,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
         case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
+        case SJVP_ERR_ROTARY: return "sjvp_rope: n must be 1..4, rot_dim even and 2 <= rot_dim <= D, and bf16 / fp16 must not be mixed";
         default: return "unknown sjvp status";
     }
 }

@@ -25,6 +25,7 @@ import torch.nn.functional as F
 from torch import Tensor, nn
 
 from .functional import safe_sdpa_jvp
+from .rotary import apply_rotary
 
 
 def math_attention(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
@@ -110,15 +111,20 @@ class DDiTBlock(nn.Module):
         nn.init.zeros_(self.adaLN_modulation.bias)
 
     def forward(self, x: Tensor, cos: Tensor, sin: Tensor, c: Tensor,
-                attention: Callable[[Tensor, Tensor, Tensor], Tensor]) -> Tensor:
+                attention: Callable[[Tensor, Tensor, Tensor], Tensor], rotary_kernel: bool = False) -> Tensor:
         B = x.shape[0]
         shift_a, scale_a, gate_a, shift_m, scale_m, gate_m = self.adaLN_modulation(c)[:, None].chunk(6, dim=2)
         h = self.norm1(x) * (1.0 + scale_a) + shift_a
         qkv = self.attn_qkv(h).view(B, self.seq_len, 3, self.n_heads, self.dim // self.n_heads)
-        q = rotate_half_embedding(qkv[:, :, 0], cos, sin)
-        k = rotate_half_embedding(qkv[:, :, 1], cos, sin)
         v = qkv[:, :, 2]
-        a = attention(q.contiguous(), k.contiguous(), v.contiguous())  # [B,S,H,D] (duo.py:141)
+        if rotary_kernel:
+            # one launch rotates q and k (and their tangents) out of the fused projection and writes
+            # the contiguous 16-bit tensors the attention kernels read
+            q, k = apply_rotary((qkv[:, :, 0], qkv[:, :, 1]), cos, sin)
+        else:
+            q = rotate_half_embedding(qkv[:, :, 0], cos, sin).contiguous()
+            k = rotate_half_embedding(qkv[:, :, 1], cos, sin).contiguous()
+        a = attention(q, k, v.contiguous())  # [B,S,H,D] (duo.py:141)
         a = a.reshape(B, self.seq_len, self.dim)
         x = self.dropout(self.attn_out(a) * gate_a) + x
         h = self.norm2(x) * (1.0 + scale_m) + shift_m
@@ -163,18 +169,24 @@ class DIT(nn.Module):
     ``F.scaled_dot_product_attention`` (duo.py:143-152); ``plain_attention`` selects that ("torch") or
     the primal-only mode of the same HIP kernels ("hip", the default).  ``attention_override`` replaces
     both with a caller-supplied function of ``(q, k, v)`` in ``[B,S,H,D]`` (the tests use
-    :func:`math_attention`).
+    :func:`math_attention`).  ``rotary`` selects the rotary embedding of q and k: "hip" (one launch
+    of the library's rotary kernel per block; GPU tensors only, there is no fallback) or "torch"
+    (:func:`rotate_half_embedding`, the separate PyTorch operations of the reference).
     """
 
     def __init__(self, vocab_size: int, hidden_size: int, cond_dim: int, n_blocks: int, n_heads: int,
                  dropout: float, length: int, plain_attention: str = "hip",
-                 attention_override: Optional[Callable[[Tensor, Tensor, Tensor], Tensor]] = None):
+                 attention_override: Optional[Callable[[Tensor, Tensor, Tensor], Tensor]] = None,
+                 rotary: str = "hip"):
         super().__init__()
         if plain_attention not in ("hip", "torch"):
             raise ValueError(f"illegal 'plain_attention': {plain_attention}")
         self.vocab_size = vocab_size
+        if rotary not in ("hip", "torch"):
+            raise ValueError(f"illegal 'rotary': {rotary}")
         self.plain_attention = plain_attention
         self.attention_override = attention_override
+        self.rotary = rotary
         self.vocab_embed = EmbeddingLayer(hidden_size, vocab_size)
         self.s_map = TimestepEmbedder(cond_dim)
         self.t_map = TimestepEmbedder(cond_dim)
@@ -201,6 +213,7 @@ class DIT(nn.Module):
         h = self.vocab_embed(x)
         cos, sin = self.rotary_emb.half_tables()
         attention = self._attention(jvp_attention)
+        rotary_kernel = self.rotary == "hip"
         for block in self.blocks:
-            h = block(h, cos, sin, cond, attention)
+            h = block(h, cos, sin, cond, attention, rotary_kernel)
         return self.output_layer(h, cond)

@@ -72,6 +72,7 @@ def main(argv=None) -> int:
     ap.add_argument("--length", type=int, default=128)
     ap.add_argument("--blocks", type=int, default=12)
     ap.add_argument("--plain-attention", choices=("hip", "torch"), default="hip")
+    ap.add_argument("--rotary", choices=("hip", "torch"), default="hip")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         print("dit_bench needs the GPU", file=sys.stderr)
@@ -79,7 +80,8 @@ def main(argv=None) -> int:
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     net = DIT(vocab_size=args.vocab, hidden_size=768, cond_dim=128, n_blocks=args.blocks, n_heads=12,
-              dropout=0.1, length=args.length, plain_attention=args.plain_attention).to(dev)
+              dropout=0.1, length=args.length, plain_attention=args.plain_attention,
+              rotary=args.rotary).to(dev)
     # the reference zero-initialises the output projection and the modulations (duo.py:124-125,188-194),
     # which makes the first step's attention gradients vanish; start from a generic point instead
     for p in net.parameters():
@@ -122,6 +124,7 @@ def main(argv=None) -> int:
         "attention_share": attn_ms / step_ms,
         "attention_launch_ms": per_kernel,
         "plain_attention": args.plain_attention,
+        "rotary": args.rotary,
         "vfm_loss": float(vf), "sd_loss": None if sd is None else float(sd),
         "max_memory_GB": torch.cuda.max_memory_allocated() / 2**30,
         "data": "synthetic (uniform token ids, random weights)",

@@ -297,3 +297,58 @@ def flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal: bool
 
 def default_scale(D: int) -> float:
     return 1.0 / math.sqrt(D)
+
+
+_ROPE_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16, torch.float32: _lib.SJVP_FP32}
+
+
+def rotary_embedding(xs: Sequence[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
+                     out_dtype: Optional[torch.dtype] = None, inverse: bool = False
+                     ) -> Tuple[torch.Tensor, ...]:
+    """Rotary position embedding of up to four ``[B,S,H,D]`` tensors of one shape and dtype in one
+    launch (``sjvp_rope``), pairing column ``i`` with ``i + rot/2`` as duo.py:45-55 does through
+    flash_attn's ``apply_rotary_emb_torch``; ``cos``/``sin`` are fp32 ``[S, rot/2]`` (any row
+    stride).  Inputs may be any views with unit last stride; the results are fresh contiguous
+    ``[B,S,H,D]`` tensors of ``out_dtype`` (default: the input dtype).  ``inverse`` applies the
+    inverse rotation (the transpose of the map, which is what back-propagates a cotangent)."""
+    xs = tuple(xs)
+    if not 1 <= len(xs) <= 4:
+        raise ValueError("rotary_embedding takes one to four tensors")
+    x0 = xs[0]
+    if not x0.is_cuda:
+        raise RuntimeError("semicat_amd kernels run on an AMD GPU only; got a tensor on "
+                           f"{x0.device} (there is no CPU fallback)")
+    out_dtype = out_dtype or x0.dtype
+    if x0.dtype not in _ROPE_DTYPES or out_dtype not in _ROPE_DTYPES:
+        raise TypeError(f"rotary_embedding supports bfloat16, float16 and float32, got {x0.dtype} -> {out_dtype}")
+    B, S, H, D = x0.shape
+    for x in xs:
+        if tuple(x.shape) != (B, S, H, D) or x.dtype != x0.dtype or x.device != x0.device:
+            raise AssertionError("rotary_embedding: all tensors must share shape, dtype and device")
+        if x.stride(-1) != 1:
+            raise AssertionError("rotary_embedding: the last dimension must have unit stride")
+    half = cos.shape[-1]
+    if cos.shape != sin.shape or cos.ndim != 2 or cos.shape[0] < S or 2 * half > D:
+        raise AssertionError(f"cos/sin must be [>= {S}, rot/2] with rot <= {D}, got {tuple(cos.shape)}")
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.stride(1) != 1 or sin.stride(1) != 1 \
+            or cos.stride(0) != sin.stride(0) or cos.device != x0.device or sin.device != x0.device:
+        raise AssertionError("cos/sin must be float32 tensors on the inputs' device with unit column "
+                             "stride and equal row strides")
+    ys = tuple(torch.empty((B, S, H, D), device=x0.device, dtype=out_dtype) for _ in xs)
+    if B * S * H == 0:
+        return ys
+    n = len(xs)
+    flat = []
+    for x, y in zip(xs, ys):  # the C ABI speaks [B,H,L,D]: (batch, head, sequence) strides
+        flat.extend((x.stride(0), x.stride(2), x.stride(1), y.stride(0), y.stride(2), y.stride(1)))
+    xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+    yp = (ctypes.c_void_p * n)(*[y.data_ptr() for y in ys])
+    lib = _lib.load()
+    with torch.cuda.device(x0.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.sjvp_rope(n, xp, yp, (ctypes.c_int64 * len(flat))(*flat), _ptr(cos), _ptr(sin),
+                           cos.stride(0), B, H, S, D, 2 * half, _ROPE_DTYPES[x0.dtype],
+                           _ROPE_DTYPES[out_dtype], 1 if inverse else 0, ctypes.c_void_p(stream))
+    _lib.check(rc)
+    return ys
+

@@ -24,6 +24,7 @@ from . import eager_backend
 
 def make_net(vocab=48, hidden=64, heads=2, blocks=2, length=16, cond=16, seed=0, **kw):
     torch.manual_seed(seed)
+    kw.setdefault("rotary", "torch")  # the CPU tests; the GPU tests ask for the HIP rotary kernel
     net = DIT(vocab_size=vocab, hidden_size=hidden, cond_dim=cond, n_blocks=blocks, n_heads=heads,
               dropout=0.0, length=length, **kw)
     # the zero-initialised modulation and output layers would make the output independent of attention
@@ -72,6 +73,8 @@ def test_state_dict_names_match_a_reference_checkpoint():
         assert names.get(n) == shape, n
     assert "blocks.0.attn_qkv.bias" not in names and "blocks.0.attn_out.bias" not in names
     fresh = DIT(30, 32, 8, 1, 2, 0.1, 8)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fresh(torch.zeros(1, 8, 30), torch.zeros(1), torch.ones(1))  # rotary="hip" needs the GPU
     assert not fresh.output_layer.linear.weight.any() and not fresh.blocks[0].adaLN_modulation.weight.any()
 
 
@@ -125,8 +128,8 @@ def _compare_steps(net, device, autocast, loss_tol, grad_tol):
     t = torch.rand(B, device=device)
     s = torch.rand(B, device=device) * t
     results = []
-    for override in (None, math_attention):
-        net.attention_override = override
+    for override, rotary in ((None, net.rotary), (math_attention, "torch")):
+        net.attention_override, net.rotary = override, rotary
         with torch.autocast(device_type=device, dtype=torch.bfloat16, enabled=autocast):
             results.append(_step_losses_and_grads(net, x0, x1, t, s))
     (vf_a, sd_a, g_a), (vf_b, sd_b, g_b) = results
@@ -153,7 +156,7 @@ def test_self_distillation_step_through_the_op_gpu():
     (configs/experiment/lm1b_dit.yaml:15), heads of 64 and sequence length 128."""
     from semicat_amd import _lib
     _lib.load()
-    net = make_net(vocab=96, hidden=128, heads=2, blocks=2, length=128, cond=32).cuda()
+    net = make_net(vocab=96, hidden=128, heads=2, blocks=2, length=128, cond=32, rotary="hip").cuda()
     _compare_steps(net, "cuda", autocast=True, loss_tol=3e-2, grad_tol=1e-1)
 
 
