@@ -317,3 +317,55 @@ def test_empty_batch_returns_empty_results(K):
     assert o.shape == to.shape == (0, 3, 128, 64)
     grads = K.attention_jvp_backward(q, q, q, q, q, q, o, to, lse, mu, dO=q, dTO=q)
     assert all(g.shape == (0, 3, 128, 64) for g in grads)
+
+
+def test_randomized_shapes_layouts_and_modes(K):
+    """A seeded sweep over shapes around the tile, stage and block boundaries (1, 31..33, 127..129,
+    255..257, ...), head dimensions, dtypes, caller layouts and cotangent modes; every output against
+    the fp64 oracle, and the primal-only forward against the fused one."""
+    import random
+    rng = random.Random(1234)
+    worst = 0.0
+    for case in range(80):
+        D = rng.choice([16, 24, 32, 48, 64, 64, 64, 80, 128])
+        Lq = rng.choice([1, 7, 16, 31, 32, 33, 64, 100, 127, 128, 129, 200, 256, 300, 385])
+        Lk = rng.choice([1, 5, 16, 31, 32, 33, 64, 96, 127, 128, 129, 255, 256, 257, 290, 352, 400])
+        B, H = rng.choice([1, 2, 3]), rng.choice([1, 2, 5])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        mode = rng.choice(["both", "both", "dO", "dTO"])
+        seq_major = rng.random() < 0.5
+        label = f"case {case}: B{B} H{H} Lq{Lq} Lk{Lk} D{D} {dtype} {mode} seq_major={seq_major}"
+        print(label, flush=True)
+        x = orc.make_inputs(B, H, Lq, Lk, D, seed=case, tangent_scale=0.3, dtype=dtype)
+        cot = {}
+        if mode != "dTO":
+            cot["dO"] = x["dO"]
+        if mode != "dO":
+            cot["dTO"] = x["dTO"]
+        ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], **cot)
+        d = {n: (t.cuda().transpose(1, 2).contiguous().transpose(1, 2) if seq_major else t.cuda())
+             for n, t in x.items()}
+        o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+        if mode == "dO":
+            g = K.attention_jvp_backward(d["q"], d["k"], d["v"], None, None, None, o, None, lse, None,
+                                         dO=d["dO"])
+        else:
+            g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                         dO=d["dO"] if mode == "both" else None, dTO=d["dTO"])
+        res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g) if t is not None}}
+        # with a single key the softmax is constant: several gradients (dq, dk and their tangent twins;
+        # dv without a cotangent on O) are zero up to the rounding of O, so the gradients are judged on
+        # the scale of the largest of them
+        floor = max(ref[m].double().norm().item() for m in GRADS if ref.get(m) is not None)
+        for n, t in res.items():
+            assert torch.isfinite(t.float()).all(), (label, n)
+            err = (t.double() - ref[n].double()).norm().item()
+            scale = ref[n].double().norm().item()
+            if Lk == 1 and n in GRADS:
+                scale = max(scale, floor)
+            assert err <= TOL_16BIT * scale, (label, n, err / max(scale, 1e-300))
+            worst = max(worst, err / max(scale, 1e-300))
+        o2, lse2 = K.attention_forward(d["q"], d["k"], d["v"])
+        assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_16BIT, label
+        assert torch.allclose(lse2[..., :Lq], lse[..., :Lq], rtol=1e-5, atol=1e-5), label
+    print(f"worst relative error over the sweep: {worst:.2e}")
