@@ -175,3 +175,34 @@ def test_plain_attention_modes_agree_gpu():
             outs[mode] = net(x, 0.5 * t, t).float()
     err = (outs["hip"] - outs["torch"]).norm() / outs["torch"].norm()
     assert err < 2e-2, err.item()
+
+
+@pytest.mark.gpu
+def test_network_under_torch_compile_gpu():
+    """The reference compiles the network (semicat.py:340-345) and keeps the op opaque to dynamo
+    (functional.py:272): with the network wrapped by torch.compile, the cross-entropy step (compiled
+    graph with a break at the op) and the self-distillation step (forward-mode AD over the wrapped
+    network) give the results of the unwrapped network.  The aot_eager backend exercises dynamo and
+    AOTAutograd without generating device code."""
+    from semicat_amd import _lib
+    _lib.load()
+    net = make_net(vocab=96, hidden=128, heads=2, blocks=2, length=128, cond=32, rotary="hip").cuda()
+    torch.manual_seed(4)
+    x1 = torch.randint(0, 96, (4, 128), device="cuda")
+    x0 = torch.randn(4, 128, 96, device="cuda")
+    t = torch.rand(4, device="cuda")
+    s = torch.rand(4, device="cuda") * t
+
+    def run(n):
+        net.zero_grad(set_to_none=True)
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            vf = ts.vfm_loss(n, x0, x1, t=t)
+            sd = ts.lag_self_distillation_loss(n, x0, x1, t=t, s=s)
+        (vf + sd).backward()
+        return vf.item(), sd.item(), net.blocks[0].attn_qkv.weight.grad.clone()
+
+    vf0, sd0, g0 = run(net)
+    torch._dynamo.reset()
+    vf1, sd1, g1 = run(torch.compile(net, backend="aot_eager"))
+    assert abs(vf1 - vf0) <= 1e-5 * abs(vf0) and abs(sd1 - sd0) <= 1e-5 * abs(sd0)
+    assert (g1 - g0).norm() <= 1e-5 * g0.norm()
