@@ -166,7 +166,7 @@ def test_library_exports_every_declared_symbol(repo_root):
     assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
     assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4
     assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4
-    for code in range(0, -9, -1):
+    for code in range(0, -10, -1):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
@@ -198,3 +198,15 @@ def test_c_abi_argument_errors_are_reported_before_any_launch():
     assert b(one, one, one, 8) == _lib.SJVP_ERR_WORKSPACE
     with pytest.raises(_lib.SjvpError):
         _lib.check(_lib.SJVP_ERR_HEAD_DIM)
+    # sjvp_rope
+    ptrs = (ctypes.c_void_p * 4)(16, 16, 16, 16)
+    rs = (ctypes.c_int64 * 24)(*([0] * 24))
+    r = lambda **kw: L.sjvp_rope(kw.get("n", 2), kw.get("x", ptrs), ptrs, rs, kw.get("cos", one), one, 32, 1, 1,
+                                 kw.get("L", 8), 64, kw.get("rot", 64), kw.get("i", 0), kw.get("o", 0), 0, None)
+    assert r(n=0) == _lib.SJVP_ERR_ROTARY and r(n=5) == _lib.SJVP_ERR_ROTARY
+    assert r(rot=63) == _lib.SJVP_ERR_ROTARY and r(rot=66) == _lib.SJVP_ERR_ROTARY and r(rot=0) == _lib.SJVP_ERR_ROTARY
+    assert r(i=0, o=1) == _lib.SJVP_ERR_ROTARY  # bf16 in, fp16 out
+    assert r(i=5) == _lib.SJVP_ERR_DTYPE
+    assert r(L=0) == _lib.SJVP_ERR_SHAPE
+    assert r(cos=None) == _lib.SJVP_ERR_NULL
+    assert r(x=(ctypes.c_void_p * 4)(16, None, 16, 16)) == _lib.SJVP_ERR_NULL
