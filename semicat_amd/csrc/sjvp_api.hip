@@ -351,6 +351,7 @@ int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* stride
     p.units = half / w + (D - rot_dim) / w;
     p.total = (int64_t)B * H * L * p.units;
     p.sign = inverse ? -1.0f : 1.0f;
+    p.h_fast = p.ys[0][1] < p.ys[0][2] ? 1 : 0;  // follow the output's memory order
     const int64_t blocks = (p.total + kRopeThreads - 1) / kRopeThreads;
     if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
 

@@ -29,6 +29,7 @@ struct RopeParams {
     int units;      // work items per row
     int64_t total;  // rows * units
     float sign;     // +1 rotation, -1 inverse rotation
+    int h_fast;     // rows are enumerated head-first (sequence-major memory) instead of position-first
 };
 
 struct F32 {};  // tag for fp32 storage (Bf16 / Fp16 are the 16-bit traits)
@@ -85,8 +86,9 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
     const int t = blockIdx.y;
     const int unit = (int)(idx % p.units);
     const int64_t row = idx / p.units;
-    const int l = (int)(row % p.L);
-    const int h = (int)((row / p.L) % p.H);
+    // consecutive rows follow the axis that is closer in memory
+    const int l = p.h_fast ? (int)((row / p.H) % p.L) : (int)(row % p.L);
+    const int h = p.h_fast ? (int)(row % p.H) : (int)((row / p.L) % p.H);
     const int64_t b = row / ((int64_t)p.L * p.H);
     const typename In::elem* x =
         reinterpret_cast<const typename In::elem*>(p.x[t]) + b * p.xs[t][0] + h * p.xs[t][1] + l * p.xs[t][2];

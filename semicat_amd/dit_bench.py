@@ -62,6 +62,32 @@ class _KernelTimer:
         return out
 
 
+def rope_only(args, dev) -> int:
+    """q and k of one block rotated out of the fused bf16 qkv projection into contiguous bf16
+    tensors: one launch reads and writes 2 * B*S*H*D 16-bit elements each way."""
+    from .dit import Rotary
+    B, S, H, D = args.batch, args.length, 12, 64
+    cos, sin = Rotary(S, D).to(dev).half_tables()
+    qkv = torch.randn(B, S, 3, H, D, device=dev).to(torch.bfloat16)
+    xs = (qkv[:, :, 0], qkv[:, :, 1])
+    for _ in range(10):
+        kernels.rotary_embedding(xs, cos, sin)
+    n = 200
+    # launches are enqueued faster than they run only for large batches; time the stream as a whole
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        kernels.rotary_embedding(xs, cos, sin)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / n * 1e3
+    nbytes = 2 * 2 * B * S * H * D * 2 + 2 * S * (D // 2) * 4
+    print(json.dumps({"workload": f"rotary embedding of q and k, B={B} S={S} H={H} D={D}, bf16 -> bf16",
+                      "us_per_launch": us, "algorithmic_bytes": nbytes, "GBps": nbytes / us / 1e3,
+                      "frac_of_8TBps": nbytes / us / 1e3 / 8000.0}))
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=64)
@@ -73,12 +99,16 @@ def main(argv=None) -> int:
     ap.add_argument("--blocks", type=int, default=12)
     ap.add_argument("--plain-attention", choices=("hip", "torch"), default="hip")
     ap.add_argument("--rotary", choices=("hip", "torch"), default="hip")
+    ap.add_argument("--rope-only", action="store_true",
+                    help="time only the rotary kernel on q and k of one block (batch x length x 12 heads of 64)")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         print("dit_bench needs the GPU", file=sys.stderr)
         return 2
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
+    if args.rope_only:
+        return rope_only(args, dev)
     net = DIT(vocab_size=args.vocab, hidden_size=768, cond_dim=128, n_blocks=args.blocks, n_heads=12,
               dropout=0.1, length=args.length, plain_attention=args.plain_attention,
               rotary=args.rotary).to(dev)
