@@ -83,6 +83,38 @@ def cpu_baseline(seconds: float = 12.0):
     }
 
 
+def measure_hardware(dev):
+    """What this GPU delivers on two plain library workloads, next to the published peaks the
+    roofline is priced against: a 1 GiB device-to-device copy (bytes read + written per second) and
+    an 8192^3 bf16 GEMM through torch.matmul."""
+    props = torch.cuda.get_device_properties(dev)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(2):
+        dst.copy_(src)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    e1.synchronize()
+    copy_gbps = 5 * 2 * src.numel() / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del src, dst
+    n = 8192
+    a_ = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    b_ = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    for _ in range(2):
+        a_ @ b_
+    e0.record()
+    for _ in range(5):
+        a_ @ b_
+    e1.record()
+    e1.synchronize()
+    gemm_tflops = 5 * 2.0 * n ** 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    return {"compute_units": props.multi_processor_count, "hbm_GiB": props.total_memory / 2 ** 30,
+            "copy_GBps": copy_gbps, "bf16_gemm_TFLOPs": gemm_tflops}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -208,6 +240,7 @@ def main() -> int:
                 dst.copy_(src)
             stream.synchronize()
 
+    hardware = measure_hardware(dev)
     ms_per_step = wall / a.steps * 1e3
     tflops = step_flops() / (ms_per_step * 1e-3) / 1e12
 
@@ -268,6 +301,7 @@ def main() -> int:
         "kernels": {n: {"ms": w["ms"], "GBps": w["GBps"], "TFLOPs": w["TFLOPs"]} for n, w in work.items()},
         "roofline": roofline,
         "device": torch.cuda.get_device_name(0),
+        "hardware": hardware,
     }
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
