@@ -35,24 +35,37 @@ def make_net(vocab=48, hidden=64, heads=2, blocks=2, length=16, cond=16, seed=0,
 
 
 def test_rotary_is_a_complex_rotation_and_relative():
+    """The real-arithmetic rotation of the product against the oracle's complex formulation, and the
+    properties that fix the oracle itself: it preserves norms, its inverse undoes it, the identity
+    slice for v, a partial rotary width, and scores that depend on the position difference only."""
+    import numpy as np
+    from oracle import rotary_oracle as ro
     torch.manual_seed(0)
     S, D = 12, 16
     rot = Rotary(S, D)
     cos, sin = rot.half_tables()
     assert cos.shape == (S, D // 2) and rot.cos_cached.shape == (1, S, 3, 1, D)
     assert torch.all(rot.cos_cached[:, :, 2] == 1) and torch.all(rot.sin_cached[:, :, 2] == 0)
+    theta = ro.rotary_angles(S, D)
+    assert np.allclose(np.cos(theta), cos.double().numpy(), atol=1e-6)  # the buffers are fp32
     x = torch.randn(2, S, 3, D, dtype=torch.float64)
-    out = rotate_half_embedding(x, cos.double(), sin.double())
-    # independent formulation: (x_i + j x_{i+D/2}) * exp(j * pos * base^(-2i/D))
-    theta = torch.arange(S, dtype=torch.float64)[:, None] * 10000.0 ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
-    z = torch.complex(x[..., : D // 2], x[..., D // 2:]) * torch.polar(torch.ones_like(theta), theta)[None, :, None, :]
-    assert torch.allclose(out, torch.cat((z.real, z.imag), -1), atol=1e-6)
+    c64, s64 = torch.from_numpy(np.cos(theta)), torch.from_numpy(np.sin(theta))
+    out = rotate_half_embedding(x, c64, s64)
+    ref = ro.rotate(x.numpy(), theta)
+    assert np.allclose(out.numpy(), ref, atol=1e-12)
+    assert np.allclose(np.linalg.norm(ref, axis=-1), np.linalg.norm(x.numpy(), axis=-1), atol=1e-12)
+    assert np.allclose(ro.rotate(ref, theta, inverse=True), x.numpy(), atol=1e-12)
+    assert np.allclose(ref[:, 0], x.numpy()[:, 0], atol=1e-12)  # position 0 is the identity
+    # partial rotary width: the columns beyond it pass through
+    part = rotate_half_embedding(x, c64[:, :4], s64[:, :4])
+    assert np.allclose(part.numpy(), ro.rotate(x.numpy(), theta[:, :4]), atol=1e-12)
+    assert torch.equal(part[..., 8:], x[..., 8:])
     # scores depend on the position difference only
-    q, k = torch.randn(D, dtype=torch.float64), torch.randn(D, dtype=torch.float64)
-    qa = rotate_half_embedding(q.expand(1, S, 1, D), cos.double(), sin.double())[0, :, 0]
-    ka = rotate_half_embedding(k.expand(1, S, 1, D), cos.double(), sin.double())[0, :, 0]
+    q, k = np.random.default_rng(0).standard_normal((2, D))
+    qa = ro.rotate(np.broadcast_to(q, (1, S, 1, D)), theta)[0, :, 0]
+    ka = ro.rotate(np.broadcast_to(k, (1, S, 1, D)), theta)[0, :, 0]
     scores = qa @ ka.T
-    assert torch.allclose(scores[3, 1], scores[9, 7], atol=1e-9) and torch.allclose(scores[0, 5], scores[6, 11], atol=1e-9)
+    assert np.isclose(scores[3, 1], scores[9, 7], atol=1e-9) and np.isclose(scores[0, 5], scores[6, 11], atol=1e-9)
 
 
 def test_state_dict_names_match_a_reference_checkpoint():

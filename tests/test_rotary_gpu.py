@@ -1,11 +1,12 @@
 """GPU tests of the rotary kernel (sjvp_rope through semicat_amd.kernels.rotary_embedding and the
-autograd function in semicat_amd.rotary) against the PyTorch restatement of the rotation in fp64
-(semicat_amd.dit.rotate_half_embedding, itself pinned on the CPU against a complex-number
-formulation).  Bars: one rounding of the output dtype (bf16 2^-8, fp16 2^-11 relative to the row
+autograd function in semicat_amd.rotary) against the oracle's complex-arithmetic rotation in fp64
+(oracle/rotary_oracle.py) and, for the two AD modes, against autograd through the PyTorch formula
+(semicat_amd.dit.rotate_half_embedding, pinned on the CPU against the same oracle).  Bars: one rounding of the output dtype (bf16 2^-8, fp16 2^-11 relative to the row
 scale) and 2e-6 for fp32 output."""
 import pytest
 import torch
 
+from oracle import rotary_oracle as ro
 from semicat_amd.dit import Rotary, rotate_half_embedding
 
 pytestmark = pytest.mark.gpu
@@ -27,8 +28,14 @@ def tables(S, rot, device="cuda"):
     return r.half_tables()  # strided views of the [1,S,3,1,rot] buffers (row stride 3*rot)
 
 
+def oracle_rotation(x, cos, sin, inverse=False):
+    """fp64 rotation of a [B,S,H,D] tensor by the angles the fp32 tables encode."""
+    theta = torch.atan2(sin.double(), cos.double()).cpu().numpy()
+    return torch.from_numpy(ro.rotate(x.double().cpu().numpy(), theta, inverse=inverse))
+
+
 def check(y, ref, dtype):
-    err = (y.double() - ref).abs().max().item()
+    err = (y.double().cpu() - ref.cpu()).abs().max().item()
     assert err <= TOL[dtype] * max(1.0, ref.abs().max().item()), (err, dtype)
 
 
@@ -46,7 +53,7 @@ def test_rotation_matches_the_fp64_formula(K, in_dtype, out_dtype, B, S, H, D, r
     yq, yk = K.rotary_embedding((q, k), cos, sin, out_dtype=out_dtype)
     assert yq.is_contiguous() and yq.dtype == out_dtype and yq.shape == (B, S, H, D)
     for x, y in ((q, yq), (k, yk)):
-        check(y, rotate_half_embedding(x.double(), cos.double(), sin.double()), out_dtype)
+        check(y, oracle_rotation(x, cos, sin), out_dtype)
     # the inverse rotation undoes it (up to the roundings of the two passes)
     back, = K.rotary_embedding((yq,), cos, sin, out_dtype=torch.float32, inverse=True)
     assert (back.double() - q.double()).abs().max().item() <= 3 * TOL[out_dtype] * max(1.0, q.abs().max().item())
@@ -59,7 +66,7 @@ def test_one_to_four_tensors_and_argument_checks(K):
     for n in (1, 3, 4):
         ys = K.rotary_embedding(xs[:n], cos, sin)
         for x, y in zip(xs, ys):
-            check(y, rotate_half_embedding(x.double(), cos.double(), sin.double()), torch.bfloat16)
+            check(y, oracle_rotation(x, cos, sin), torch.bfloat16)
     with pytest.raises(ValueError):
         K.rotary_embedding(xs + xs[:1], cos, sin)
     with pytest.raises(AssertionError):
