@@ -369,3 +369,55 @@ def test_randomized_shapes_layouts_and_modes(K):
         assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_16BIT, label
         assert torch.allclose(lse2[..., :Lq], lse[..., :Lq], rtol=1e-5, atol=1e-5), label
     print(f"worst relative error over the sweep: {worst:.2e}")
+
+
+def test_graph_replays_match_eager_launches(K):
+    """The launches are capturable in a HIP graph (no allocation, no memset, no host synchronisation
+    inside the library): three replays, with the program's own eager work and synchronisations between
+    them and fresh inputs copied in before each, equal the eager results bit for bit."""
+    B, H, L, D = 2, 3, 128, 64
+    names = orc.TENSOR_ORDER
+    sets = [orc.make_inputs(B, H, L, L, D, seed=20 + i, dtype=torch.bfloat16) for i in range(3)]
+    d = {n: torch.empty_like(sets[0][n], device="cuda") for n in names}
+    Lr = K.stat_rows(L)
+    o, to = torch.empty_like(d["q"]), torch.empty_like(d["q"])
+    lse = torch.empty((B, H, Lr), device="cuda", dtype=torch.float32)
+    mu = torch.empty_like(lse)
+    grads = tuple(torch.empty_like(d["q"]) for _ in range(6))
+    from semicat_amd import _lib
+    ws = torch.empty((_lib.load().sjvp_bwd_workspace_bytes(B, H, L, L, D, _lib.SJVP_BF16),), device="cuda",
+                     dtype=torch.uint8)
+
+    def step():
+        K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o=o, to=to, lse=lse, mu=mu,
+                                with_li=False)
+        K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"], grads=grads, workspace=ws)
+
+    def load(i):
+        for n in names:
+            d[n].copy_(sets[i][n])
+
+    eager = []
+    for i in range(3):
+        load(i)
+        step()
+        torch.cuda.synchronize()
+        eager.append([t.clone() for t in (o, to, lse, mu, *grads)])
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        load(0)
+        step()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+        for i in (1, 2, 0):
+            load(i)
+            for t in (o, to, *grads):
+                t.zero_()  # eager work between the replays
+            stream.synchronize()
+            graph.replay()
+            stream.synchronize()
+            for got, want in zip((o, to, lse, mu, *grads), eager[i]):
+                assert torch.equal(got, want), f"replay on input set {i} differs from the eager launch"
