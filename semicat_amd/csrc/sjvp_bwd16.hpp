@@ -322,11 +322,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             if (do_q) {
                 a0 += a1;
                 u32x2 val = {T::pack2(a0[0] * p.scale, a0[1] * p.scale), T::pack2(a0[2] * p.scale, a0[3] * p.scale)};
-                *reinterpret_cast<u32x2*>(p.dq.head(b, h) + (int64_t)qrow * p.dq.sl + col) = val;
+                __builtin_nontemporal_store(val, reinterpret_cast<u32x2*>(p.dq.head(b, h) + (int64_t)qrow * p.dq.sl + col));
             }
             if (do_t) {
                 u32x2 val = {T::pack2(a2[0] * p.scale, a2[1] * p.scale), T::pack2(a2[2] * p.scale, a2[3] * p.scale)};
-                *reinterpret_cast<u32x2*>(p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl + col) = val;
+                __builtin_nontemporal_store(val, reinterpret_cast<u32x2*>(p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl + col));
             }
         }
     };

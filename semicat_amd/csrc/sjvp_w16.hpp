@@ -205,7 +205,10 @@ __device__ __forceinline__ void store_tile16(elem_t* stage, elem_t* gp, int64_t 
         const int c = lane % CH;
         if (RPI <= 16 || r < 16) {
             const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * P + 8 * c);
-            if (row0 + r < L && 8 * c < D) *reinterpret_cast<u32x4*>(gp + (int64_t)(row0 + r) * sl + 8 * c) = v;
+            if (row0 + r < L && 8 * c < D) {
+                u32x4* dst = reinterpret_cast<u32x4*>(gp + (int64_t)(row0 + r) * sl + 8 * c);
+                __builtin_nontemporal_store(v, dst);  // written once, not read again by this launch
+            }
         }
     }
 }
