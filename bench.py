@@ -7,7 +7,9 @@ A step is one pass of the hot path over one batch: the fused forward (O, TO, lse
 the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
 B=64, H=12, L=128, D=64, bf16 inputs / fp32 accumulation, q,k,v ~ N(0,1)*0.5, tangents ~ N(0,1)*0.1,
 cotangents ~ N(0,1), seed 0, inputs resident in HBM.  Throughput uses the work model
-42*B*H*L^2*D flop per step (forward 6 + backward 15 tile contractions).  Prints ONE JSON line.
+42*B*H*L^2*D flop per step (forward 6 + backward 15 tile contractions).  The GPU is first kept busy
+for 0.3 s (untimed) so that its clocks have settled, then W warmup steps run, then exactly K steps are
+timed.  Prints ONE JSON line.
 """
 from __future__ import annotations
 
@@ -32,8 +34,8 @@ NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
 # kernel of --calib-copy: one FETCH_SIZE unit is 2 KiB, one WRITE_SIZE unit 1 KiB there).
 MEASURED_TRAFFIC_BYTES = {
-    "fwd16_kernel": (2 * 36937.3 + 25346.8) * 1024,
-    "bwd_fused16_kernel": (2 * 61936.5 + 87018.5) * 1024,
+    "fwd16_kernel": (2 * 36937.0 + 25346.7) * 1024,
+    "bwd_fused16_kernel": (2 * 61937.0 + 86485.5) * 1024,
 }
 
 
@@ -118,8 +120,8 @@ def measure_hardware(dev):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--graph", action="store_true",
                     help="replay a HIP graph of one step instead of launching through the C ABI every step")
     ap.add_argument("--no-graph", action="store_true", help="(default behaviour; kept for old command lines)")
@@ -166,9 +168,14 @@ def main() -> int:
             fwd()
             bwd()
 
-        for _ in range(3):
-            step()
-        stream.synchronize()
+        # Bring the GPU out of its idle power state before anything is timed: a step lasts tens of
+        # microseconds, and the clocks take some hundred milliseconds of load to settle (with 20 warmup
+        # steps the same kernels measure 10 % slower than in steady state).
+        t_ramp = time.perf_counter() + 0.3
+        while time.perf_counter() < t_ramp:
+            for _ in range(50):
+                step()
+            stream.synchronize()
         if a.graph:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
