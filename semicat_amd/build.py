@@ -10,7 +10,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libsjvp.so")
 SOURCES = [os.path.join(CSRC, "sjvp_api.hip")]
-HEADERS = [os.path.join(CSRC, n) for n in ("sjvp_device.hpp", "sjvp_fwd.hpp", "sjvp_bwd.hpp")] + [
+HEADERS = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith(".hpp")) + [
     os.path.join(os.path.dirname(PKG_DIR), "include", "sjvp.h")]
 
 HIPCC_FLAGS = [
