@@ -63,7 +63,12 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int g = lane >> 4;
-    const int bh = blockIdx.x;
+    // Heads are taken in descending order, groups of eight kept together (workgroups are dealt to
+    // the eight XCDs round-robin, and the forward takes head i in workgroup i): when the backward
+    // directly follows the forward, the heads the forward touched last are still in their XCD's L2.
+    const int groups = (int)gridDim.x >> 3;
+    const int bh = (int)blockIdx.x < 8 * groups ? 8 * (groups - 1 - ((int)blockIdx.x >> 3)) + ((int)blockIdx.x & 7)
+                                                : (int)blockIdx.x;
     const int b = bh / p.H, h = bh % p.H;
     const int key_slabs = (p.Lk + 31) >> 5;           // 32-key slabs that hold at least one key
     const bool wave_active = (wave >> 1) < key_slabs;  // waves of a partly filled slab all take part
