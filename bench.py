@@ -34,8 +34,8 @@ NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
 # kernel of --calib-copy: one FETCH_SIZE unit is 2 KiB, one WRITE_SIZE unit 1 KiB there).
 MEASURED_TRAFFIC_BYTES = {
-    "fwd16_kernel": (2 * 36937.5 + 25347.0) * 1024,
-    "bwd_fused16_kernel": (2 * 61936.5 + 90100.9) * 1024,
+    "fwd16_kernel": (2 * 36937.5 + 25344.4) * 1024,
+    "bwd_fused16_kernel": (2 * 61934.8 + 73985.3) * 1024,
 }
 
 

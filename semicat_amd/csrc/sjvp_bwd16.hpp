@@ -9,9 +9,10 @@
 //      registers, keys in lanes); dK, dV, dK_dot, dV_dot accumulate in registers; dS and dS_dot go
 //      as 16-bit into an LDS bounce tile [key][query];
 //   3. after a barrier, wave w forms one 16x16 tile of dQ and one of dQ_dot for the stage from the
-//      bounce tile and the own rows of K, K_dot (both through transposing LDS reads) and stores
-//      them: a stage's dQ rows are complete after one pass over the keys, so nothing is accumulated
-//      across stages and no atomics or partial sums are needed.
+//      bounce tile and the own rows of K, K_dot (both through transposing LDS reads) and puts them
+//      into a staging tile, from where 512 threads send the stage's dQ / dQ_dot rows out as whole
+//      rows after the next barrier: a stage's dQ rows are complete after one pass over the keys, so
+//      nothing is accumulated across stages and no atomics or partial sums are needed.
 // Results are deterministic.
 #pragma once
 #include "sjvp_bwd.hpp"
@@ -21,7 +22,8 @@ namespace sjvp {
 
 // LDS layout: [own K, K_dot: four slabs each][own V, V_dot: four slabs each; once they have been
 // read into registers the same memory is the bounce tile dS (, dS_dot): [128 keys][32 queries + pad]]
-// [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d][sink]
+// [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d]
+// [staging tile of a stage's dQ (, dQ_dot)][sink]
 // After the last stage the ring doubles as the per-wave staging tiles of the output stores.
 template <int HD, int R, bool HAS_DO, bool HAS_G>
 struct Fused16Smem {
@@ -34,7 +36,10 @@ struct Fused16Smem {
     static constexpr int bounce_one = kOwned16 * bpitch;
     static constexpr int bounce = (HAS_G ? 2 : 1) * bounce_one;
     static constexpr int vregion = own_v > bounce ? own_v : bounce;
-    static constexpr int sink = (own_k + vregion + R * slot) * (int)sizeof(elem_t);
+    // staging of a stage's dQ (, dQ_dot) tiles, [32 queries][HD + 8], so that they leave as whole rows
+    static constexpr int qpitch = HD + 8;
+    static constexpr int qstage = (HAS_G ? 2 : 1) * kStageRows * qpitch;
+    static constexpr int sink = (own_k + vregion + R * slot + qstage) * (int)sizeof(elem_t);
     static constexpr int bytes = sink + kSink16;
     static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
@@ -50,6 +55,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     elem_t* bounceS = ownV;                               // aliases V, V_dot after the prologue
     elem_t* bounceT = ownV + SM::bounce_one;
     elem_t* ring = ownV + SM::vregion;
+    elem_t* qstage = ring + R * SM::slot;                 // dQ (, dQ_dot) tiles of one stage on their way out
     // slot layout
     constexpr int oTQ = SE, oG = 2 * SE, oDO = (HAS_G ? 3 : 1) * SE;
     constexpr int oO = oDO + (HAS_DO ? SE : 0), oTO = oO + SE;
@@ -320,19 +326,32 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         } else {
             for (int kk = 0; kk < key_slabs; ++kk) step(kk);
         }
-        // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3
-        const int qrow = row0 + 16 * qt + n;
-        const int col = 16 * dt + 4 * g;
-        if (qrow < p.Lq && col < p.D) {
-            if (do_q) {
-                a0 += a1;
-                u32x2 val = {T::pack2(a0[0] * p.scale, a0[1] * p.scale), T::pack2(a0[2] * p.scale, a0[3] * p.scale)};
-                __builtin_nontemporal_store(val, reinterpret_cast<u32x2*>(p.dq.head(b, h) + (int64_t)qrow * p.dq.sl + col));
-            }
-            if (do_t) {
-                u32x2 val = {T::pack2(a2[0] * p.scale, a2[1] * p.scale), T::pack2(a2[2] * p.scale, a2[3] * p.scale)};
-                __builtin_nontemporal_store(val, reinterpret_cast<u32x2*>(p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl + col));
-            }
+        // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3: into the staging tile, from
+        // where flush_rows() sends whole rows after the next barrier
+        elem_t* st = qstage + (16 * qt + n) * SM::qpitch + 16 * dt + 4 * g;
+        if (do_q) {
+            a0 += a1;
+            *reinterpret_cast<u32x2*>(st) =
+                u32x2{T::pack2(a0[0] * p.scale, a0[1] * p.scale), T::pack2(a0[2] * p.scale, a0[3] * p.scale)};
+        }
+        if (do_t) {
+            *reinterpret_cast<u32x2*>(st + kStageRows * SM::qpitch) =
+                u32x2{T::pack2(a2[0] * p.scale, a2[1] * p.scale), T::pack2(a2[2] * p.scale, a2[3] * p.scale)};
+        }
+    };
+    // dQ (threads 0..255) and dQ_dot (256..511) of the stage that starts at row0: one 16-byte piece
+    // of a row per thread (HD / 8 pieces per row).  Issued before the stage copy of the iteration, so
+    // the stores are older than every copy a later wait_stages() still allows to be outstanding.
+    auto flush_rows = [&](int row0) {
+        constexpr int CH = HD / 8;
+        const int half = tid >> 8, t = tid & 255;
+        if (half == 1 && !HAS_G) return;
+        const int r = t / CH, c = t % CH;
+        if (r < kStageRows && row0 + r < p.Lq && 8 * c < p.D) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(qstage + half * kStageRows * SM::qpitch + r * SM::qpitch + 8 * c);
+            elem_t* dst = (half == 0 ? p.dq.head(b, h) + (int64_t)(row0 + r) * p.dq.sl
+                                     : p.dtq.head(b, h) + (int64_t)(row0 + r) * p.dtq.sl) + 8 * c;
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
         }
     };
 
@@ -356,6 +375,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
         __syncthreads();
+        if (i >= 1) flush_rows((i - 1) * kStageRows);
         if (issued < ns && issued < i + R) issue_next();  // into the slot of stage issued - R <= i - 1
         elem_t* slot = ring + (i % R) * SM::slot;
         if (wave_active) tile(slot);
@@ -366,6 +386,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         else row_outputs(i * kStageRows, std::false_type{});
     }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    flush_rows((ns - 1) * kStageRows);
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = wave * 16;
