@@ -60,8 +60,12 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     const int n = lane & 15;
     const int g = lane >> 4;
     const int q_blocks = p.Lr / kXOwned16;  // statistic rows up to Lr are all covered
-    const int bh = blockIdx.x / q_blocks;
-    const int qb = blockIdx.x % q_blocks;
+    // Workgroups run through the heads in descending order: this launch follows the forward, which
+    // ran through them in ascending order, so it starts on what the caches still hold (the
+    // column-owned launch after it ascends again).
+    const int bid = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int bh = bid / q_blocks;
+    const int qb = bid % q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const int q0 = qb * kXOwned16;
     const int qrow = q0 + wave * 16 + n;
