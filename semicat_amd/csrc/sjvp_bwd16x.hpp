@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     // Workgroups run through the heads in descending order: this launch follows the forward, which
     // ran through them in ascending order, so it starts on what the caches still hold (the
     // column-owned launch after it ascends again).
-    const int bid = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int bid = (int)gridDim.x - 1 - xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
     const int bh = bid / q_blocks;
     const int qb = bid % q_blocks;
     const int b = bh / p.H, h = bh % p.H;
@@ -243,8 +243,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     const int n = lane & 15;
     const int g = lane >> 4;
     const int k_blocks = (p.Lk + kXOwned16 - 1) / kXOwned16;
-    const int bh = blockIdx.x / k_blocks;
-    const int kb = blockIdx.x % k_blocks;
+    const int bid = xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
+    const int bh = bid / k_blocks;
+    const int kb = bid % k_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const int key0 = kb * kXOwned16;
     const int krow = key0 + wave * 16 + n;

@@ -46,8 +46,11 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;  // owned query within the wave
     const int g = lane >> 4;  // lane group
-    const int bh = blockIdx.x / p.q_blocks;
-    const int qb = blockIdx.x % p.q_blocks;
+    // with one workgroup per (batch, head) the identity is kept: the fused backward relies on head i
+    // having run on XCD i % 8
+    const int bid = p.q_blocks > 1 ? xcd_linear_id((int)blockIdx.x, (int)gridDim.x) : (int)blockIdx.x;
+    const int bh = bid / p.q_blocks;
+    const int qb = bid % p.q_blocks;
     const int b = bh / p.H, h = bh % p.H;
     const int q0 = qb * kOwned16;
     const int qrow = q0 + wave * 16 + n;

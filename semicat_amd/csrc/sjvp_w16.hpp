@@ -26,6 +26,16 @@ struct Src {
     int64_t sl;         // row stride in elements
 };
 
+// Workgroups are dealt to the eight XCDs round-robin (workgroup i runs on XCD i % 8), each XCD with
+// an L2 of its own.  Kernels in which several workgroups of a (batch, head) pair stream the same
+// rows take their work item from this map: XCD x gets the contiguous range x * G/8 .. (x+1) * G/8 - 1
+// of the linear order, so the workgroups of one pair run on one XCD, close in time, and find the
+// streamed rows in its L2.  Grids that are not a multiple of eight keep the identity.
+__device__ __forceinline__ int xcd_linear_id(int bid, int grid) {
+    if (grid & 7) return bid;
+    return (bid & 7) * (grid >> 3) + (bid >> 3);
+}
+
 // Per-thread geometry of an LDS-DMA copy of NS slabs that lie back to back in LDS: slab j holds rows
 // 32*(j % SPTN) .. +31 (relative to the first row of the copy window) of tensor j / SPTN.  Successive
 // calls of issue() copy successive windows (32*SPTN rows further down every tensor).  Every wave
