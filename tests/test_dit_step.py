@@ -104,6 +104,10 @@ def test_interpolate_and_losses_against_direct_evaluation():
     logits = net(xt, t, t)
     direct = -(torch.log_softmax(logits, -1).gather(-1, x1[..., None])).mean()
     assert torch.allclose(loss, direct, atol=1e-5)
+    # the reference's formulation (class axis second), also with label smoothing
+    assert torch.allclose(loss, F.cross_entropy(logits.transpose(-1, 1), x1), atol=1e-6)
+    assert torch.allclose(ts.vfm_loss(net, x0, x1, label_smoothing=0.1, t=t),
+                          F.cross_entropy(logits.transpose(-1, 1), x1, label_smoothing=0.1), atol=1e-6)
     # the time derivative inside the self-distillation loss against a central difference in fp64
     net64 = make_net(attention_override=math_attention).double()
     s = torch.rand(B, dtype=torch.float64) * t.double()
