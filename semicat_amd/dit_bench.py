@@ -92,6 +92,54 @@ def rope_only(args, dev) -> int:
     return 0
 
 
+def graph_step(args, net, opt, x1) -> int:
+    """The whole step captured once and replayed: forward-mode AD through the network, the attention
+    and rotary launches of the library, the backward and AdamW all become nodes of one HIP graph (the
+    library allocates nothing, records no memset and never synchronises, so its launches can be
+    captured).  The replay time is what the kernels of a step take without the host issuing them one
+    by one.  The random draws of a step come from the default generator, which graph capture
+    advances per replay."""
+    def step():
+        opt.zero_grad(set_to_none=False)
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            vf, sd = train_step.model_step(net, x1, (args.length, args.vocab), sd_prop=args.sd_prop)
+        loss = vf if sd is None else (sd if int(args.sd_prop * args.batch) == args.batch else vf + sd)
+        loss.backward()
+        opt.step()
+        return vf.detach(), None if sd is None else sd.detach()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(3, args.warmup)):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        vf, sd = step()
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    print(json.dumps({
+        "workload": f"LM1B DiT step: {args.blocks} blocks, width 768, 12x64 heads, seq {args.length}, "
+                    f"vocab {args.vocab}, batch {args.batch}, sd_prop {args.sd_prop}, bf16 autocast, AdamW",
+        "launch": "HIP graph replay of one whole step",
+        "ms_per_step": e0.elapsed_time(e1) / args.steps,
+        "plain_attention": args.plain_attention, "rotary": args.rotary,
+        "vfm_loss": float(vf), "sd_loss": None if sd is None else float(sd),
+        "max_memory_GB": torch.cuda.max_memory_allocated() / 2**30,
+        "data": "synthetic (uniform token ids, random weights)",
+    }))
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=64)
@@ -103,6 +151,8 @@ def main(argv=None) -> int:
     ap.add_argument("--blocks", type=int, default=12)
     ap.add_argument("--plain-attention", choices=("hip", "torch"), default="hip")
     ap.add_argument("--rotary", choices=("hip", "torch"), default="hip")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one whole step (losses, backward, AdamW) in a HIP graph and time its replays")
     ap.add_argument("--rope-only", action="store_true",
                     help="time only the rotary kernel on q and k of one block (batch x length x 12 heads of 64)")
     args = ap.parse_args(argv)
@@ -121,9 +171,12 @@ def main(argv=None) -> int:
     for p in net.parameters():
         if not p.any():
             torch.nn.init.normal_(p, std=0.02)
-    opt = torch.optim.AdamW(net.parameters(), lr=1e-4, weight_decay=0.0)
+    opt = torch.optim.AdamW(net.parameters(), lr=1e-4, weight_decay=0.0, capturable=args.graph)
     gen = torch.Generator(device=dev).manual_seed(0)
     x1 = torch.randint(0, args.vocab, (args.batch, args.length), device=dev, generator=gen)
+
+    if args.graph:
+        return graph_step(args, net, opt, x1)
 
     def step():
         opt.zero_grad(set_to_none=True)
