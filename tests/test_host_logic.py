@@ -210,3 +210,14 @@ def test_c_abi_argument_errors_are_reported_before_any_launch():
     assert r(L=0) == _lib.SJVP_ERR_SHAPE
     assert r(cos=None) == _lib.SJVP_ERR_NULL
     assert r(x=(ctypes.c_void_p * 4)(16, None, 16, 16)) == _lib.SJVP_ERR_NULL
+
+
+def test_companion_benchmarks_refuse_to_run_without_gpu(capsys):
+    """The companion benchmarks measure the HIP path only: without a GPU they say so and return 2."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from semicat_amd import dit_bench, shape_bench
+    assert shape_bench.main(["--shape", "2", "2", "64", "64"]) == 2
+    assert dit_bench.main([]) == 2
+    assert "needs the GPU" in capsys.readouterr().err
