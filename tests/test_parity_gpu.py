@@ -171,6 +171,24 @@ def test_unaligned_and_odd_head_dim_take_the_scalar_path(K):
     assert_parity(res, ref, TOL_16BIT, label="misaligned")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Lq,Lk,D,ps", [(2, 2, 128, 128, 64, 5.0), (1, 2, 200, 300, 64, 4.0),
+                                            (1, 2, 96, 160, 128, 3.0), (1, 1, 128, 128, 64, 8.0)])
+def test_large_logits(K, dtype, B, H, Lq, Lk, D, ps):
+    """q, k ~ ps * N(0,1): scaled scores reach +-100 (ps = 5) to +-270 (ps = 8), where exp() of an
+    unshifted score overflows fp32 and every softmax row is close to one-hot.  Everything must stay
+    finite; the parity gate holds up to ps = 5 (at ps = 8 the bf16 rounding of the score tangents,
+    which grow with ps^2, dominates and the gate is relaxed to 2e-2)."""
+    x = orc.make_inputs(B, H, Lq, Lk, D, seed=5, primal_scale=ps, tangent_scale=0.1, dtype=dtype)
+    x["v"] = (x["v"].float() / ps).to(dtype)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    for n in OUTS + ("lse", "mu"):
+        assert torch.isfinite(res[n].float()).all(), n
+    assert res["lse"].max() > 30.0
+    assert_parity(res, ref, TOL_16BIT if ps <= 5.0 else 2e-2, label=f"large logits {dtype} ps={ps}")
+
+
 def test_bitwise_determinism(K):
     x = orc.make_inputs(2, 2, 200, 136, 64, seed=7, dtype=torch.bfloat16)
     a = run_hip(K, x)
