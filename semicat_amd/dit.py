@@ -124,7 +124,8 @@ class DDiTBlock(nn.Module):
         else:
             q = rotate_half_embedding(qkv[:, :, 0], cos, sin).contiguous()
             k = rotate_half_embedding(qkv[:, :, 1], cos, sin).contiguous()
-        a = attention(q, k, v.contiguous())  # [B,S,H,D] (duo.py:141)
+        # v stays a strided view of the fused projection: the attention kernels read through strides
+        a = attention(q, k, v if rotary_kernel else v.contiguous())  # [B,S,H,D] (duo.py:141)
         a = a.reshape(B, self.seq_len, self.dim)
         x = self.dropout(self.attn_out(a) * gate_a) + x
         h = self.norm2(x) * (1.0 + scale_m) + shift_m
