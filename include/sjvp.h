@@ -20,7 +20,8 @@
  *   - dtype: SJVP_BF16 or SJVP_FP16 for every tensor; accumulation and softmax are fp32.
  *   - Row statistics lse / mu / li are fp32 [B,H,Lr] contiguous with Lr = ceil(Lq/128)*128
  *     (ryu_triton.py:351-358); rows >= Lq receive log(Lk), 0, Lk.
- *   - scale <= 0 selects the default 1/sqrt(D) (ryu_triton.py:324-325).
+ *   - scale == 0 selects the default 1/sqrt(D) (ryu_triton.py:324-325); a negative or non-finite
+ *     scale is an error.
  *   - The caller owns every buffer, including the workspace; the library allocates no device
  *     memory, keeps no pointer after returning, has no mutable global state, enqueues on the given
  *     hipStream_t (passed as void*) of the CURRENT device and returns without synchronising.
@@ -49,10 +50,11 @@ enum sjvp_status {
     SJVP_ERR_HEAD_DIM = -3,  /* D < 16 (ryu_triton.py:319-322) or D > 128 (flash_jvp_backward.py:2318) */
     SJVP_ERR_DTYPE = -4,     /* dtype is neither SJVP_BF16 nor SJVP_FP16                     */
     SJVP_ERR_WORKSPACE = -5, /* workspace NULL or smaller than sjvp_bwd_workspace_bytes()    */
-    SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (hipGetLastError)           */
+    SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (status of hipLaunchKernel) */
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
     SJVP_ERR_PARTS = -8,     /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
-    SJVP_ERR_ROTARY = -9     /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16 */
+    SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16 */
+    SJVP_ERR_SCALE = -10     /* scale negative, infinite or NaN (0 selects the default)      */
 };
 
 /* Indices into the stride tables: strides[3*i + {0,1,2}] = (batch, head, sequence) strides in
@@ -136,6 +138,10 @@ const char* sjvp_strerror(int status);
 
 /* SJVP_VERSION the library was built with. */
 int sjvp_version(void);
+
+/* "SJVP_BUILD_ID=<hash>": identifies the sources this binary was built from, so that a host layer
+ * can refuse a stale library.  No counterpart in the reference. */
+const char* sjvp_build_id(void);
 
 #ifdef __cplusplus
 }

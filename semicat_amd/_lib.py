@@ -3,7 +3,6 @@ missing or a call fails, an exception is raised."""
 from __future__ import annotations
 
 import ctypes
-import os
 import threading
 
 from . import build as _build
@@ -22,6 +21,7 @@ SJVP_ERR_LAUNCH = -6
 SJVP_ERR_COTANGENT = -7
 SJVP_ERR_PARTS = -8
 SJVP_ERR_ROTARY = -9
+SJVP_ERR_SCALE = -10
 
 SJVP_BWD_ROW = 1
 SJVP_BWD_COL = 2
@@ -32,7 +32,7 @@ B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
 EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_workspace_bytes", "sjvp_rope",
-           "sjvp_strerror", "sjvp_version")
+           "sjvp_strerror", "sjvp_version", "sjvp_build_id")
 
 _lock = threading.Lock()
 _lib = None
@@ -45,14 +45,15 @@ class SjvpError(RuntimeError):
 
 
 def load() -> ctypes.CDLL:
-    """Load the in-tree shared library (building it first only if it does not exist)."""
+    """Load the in-tree shared library; it is built first when it does not exist or is older than one
+    of its sources (a stale binary is never loaded silently)."""
     global _lib
     if _lib is not None:
         return _lib
     with _lock:
         if _lib is None:
             path = _build.LIB_PATH
-            if not os.path.exists(path):
+            if _build.is_stale():
                 _build.build()
             lib = ctypes.CDLL(path)
             vp, fp, i, i64p = ctypes.c_void_p, ctypes.POINTER(ctypes.c_float), ctypes.c_int, \
@@ -73,6 +74,10 @@ def load() -> ctypes.CDLL:
             lib.sjvp_strerror.restype = ctypes.c_char_p
             lib.sjvp_version.argtypes = []
             lib.sjvp_version.restype = i
+            lib.sjvp_build_id.argtypes = []
+            lib.sjvp_build_id.restype = ctypes.c_char_p
+            if lib.sjvp_build_id().decode() != "SJVP_BUILD_ID=" + _build.source_id():
+                raise RuntimeError(f"{path} was built from other sources than the ones in this tree")
             _lib = lib
     return _lib
 

@@ -5,12 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
-#include "sjvp_bwd.hpp"
-#include "sjvp_bwd16.hpp"
-#include "sjvp_bwd16x.hpp"
-#include "sjvp_fwd.hpp"
-#include "sjvp_fwd16.hpp"
+#include "sjvp_launch.hpp"
 #include "sjvp_rope.hpp"
+#include "sjvp_w16.hpp"
 
 using namespace sjvp;
 
@@ -35,156 +32,24 @@ inline OutView out_view(void* p, const int64_t* s) {
     return OutView{static_cast<elem_t*>(p), s[0], s[1], s[2]};
 }
 
-int check_common(int B, int H, int Lq, int Lk, int D, int dtype) {
+int check_common(int B, int H, int Lq, int Lk, int D, int dtype, float scale) {
     if (dtype != SJVP_BF16 && dtype != SJVP_FP16) return SJVP_ERR_DTYPE;
     if (B < 1 || H < 1 || Lq < 1 || Lk < 1) return SJVP_ERR_SHAPE;
     if (D < 16 || D > 128) return SJVP_ERR_HEAD_DIM;
     const int64_t blocks = (int64_t)B * H * ((int64_t)round_up(Lq > Lk ? Lq : Lk, 32) / 32);
     if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
+    if (!(scale >= 0.f) || isinf(scale)) return SJVP_ERR_SCALE;  // 0 selects the default; NaN fails too
     return SJVP_OK;
 }
 
-template <typename K, typename... Extra>
-int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params, int threads,
-           Extra... extra) {
-    if (smem_bytes > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                smem_bytes) != hipSuccess) {
-            (void)hipGetLastError();
-            return SJVP_ERR_LAUNCH;
-        }
-    }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), smem_bytes, stream, params, extra...);
-    return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
-}
+inline float resolve_scale(float scale, int D) { return scale > 0.f ? scale : 1.0f / sqrtf((float)D); }
 
-template <typename K>
-int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const auto& params) {
-    return launch(kernel, grid, smem_bytes, stream, params, kThreads);
-}
-
-// Ring depths (stages of 32 rows in flight) of the 16-wide kernels per head-dimension class, sized
-// to the LDS a workgroup may take when several of them are to share the 160 KB of a CU.
-template <int HD>
-struct Ring {
-    static constexpr int fwd16 = 2;                    // with tangents (four slabs per stage)
-    static constexpr int fwd16_primal = 4;             // primal only (two slabs per stage)
-    static constexpr int fused = 3;
-    static constexpr int pair = HD == 128 ? 2 : 3;     // row-owned / column-owned backward pair
-};
-
-// key-axis length from which the forward takes two stages per barrier
-constexpr int kFwdPairedFrom = 256;
-
-// 32-wide forward for inputs of any alignment (register-staged copies, one stage in LDS)
-template <typename T, int HD>
-int fwd_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    if (jvp) return launch(fwd_kernel<T, HD, true>, grid, FwdSmem<HD, true>::bytes, stream, p);
-    return launch(fwd_kernel<T, HD, false>, grid, FwdSmem<HD, false>::bytes, stream, p);
-}
-
-template <typename T, int HD>
-int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    // two stages in flight and at most 128 registers: two workgroups (sixteen waves) share a CU, which
-    // overlaps one's copies with the other's arithmetic; HD = 128 needs the whole register budget
-    constexpr int R = Ring<HD>::fwd16;
-    constexpr int RP = Ring<HD>::fwd16_primal;
-    constexpr int OCC = HD == 128 ? 2 : 4;
-    if (p.Lk >= kFwdPairedFrom) {
-        // long key axes: two stages per barrier over a ring of four slots in the same LDS footprint
-        if (jvp)
-            return launch(fwd16_kernel<T, HD, 4, true, OCC, 2>, grid, Fwd16Smem<HD, 4, true, 2>::bytes, stream,
-                          p, kThreads16);
-        return launch(fwd16_kernel<T, HD, 4, false, OCC, 2>, grid, Fwd16Smem<HD, 4, false, 2>::bytes, stream,
-                      p, kThreads16);
-    }
-    if (jvp)
-        return launch(fwd16_kernel<T, HD, R, true, OCC>, grid, Fwd16Smem<HD, R, true>::bytes, stream, p,
-                      kThreads16);
-    return launch(fwd16_kernel<T, HD, RP, false, OCC>, grid, Fwd16Smem<HD, RP, false>::bytes, stream, p,
-                  kThreads16);
-}
-
+// Kernel selection of the backward: the single launch where it fits, else the row + column pair.
 template <typename T>
-int fwd_dtype(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
-    // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
-    if (p.vec) {
-        if (p.D <= 32) return fwd16_hd<T, 32>(p, grid, jvp, stream);
-        if (p.D <= 64) return fwd16_hd<T, 64>(p, grid, jvp, stream);
-        return fwd16_hd<T, 128>(p, grid, jvp, stream);
-    }
-    if (p.D <= 32) return fwd_hd<T, 32>(p, grid, jvp, stream);
-    if (p.D <= 64) return fwd_hd<T, 64>(p, grid, jvp, stream);
-    return fwd_hd<T, 128>(p, grid, jvp, stream);
-}
-
-template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DMA>
-int bwd_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
-    if constexpr (DMA) {
-        if constexpr (HD <= 64) {
-            // short key axis: one launch, one workgroup per (batch, head)
-            if (parts == SJVP_BWD_ALL && p.Lk <= kOwned16) {
-                constexpr int FR = Ring<HD>::fused;
-                return launch(bwd_fused16_kernel<T, HD, FR, HAS_DO, HAS_G>, BH,
-                              Fused16Smem<HD, FR, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
-            }
-        }
-        // 16-wide pair: the row-owned kernel first (besides dQ, dQ_dot it leaves the row sums in the
-        // workspace), then the column-owned one; workgroups of four waves own 64 positions
-        constexpr int XR = Ring<HD>::pair;
-        int rc = SJVP_OK;
-        if (parts & SJVP_BWD_ROW)
-            rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, (HD == 128 ? 2 : 3)>,
-                        BH * (p.Lr / kXOwned16), Row16Smem<HD, XR, HAS_G>::bytes, stream, p, kXThreads16);
-        if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
-        const int grid = BH * ((p.Lk + kXOwned16 - 1) / kXOwned16);
-        using CS = Col16Smem<HD, XR, HAS_DO, HAS_G>;
-        if constexpr (HD == 128) {
-            // two launches, each accumulating two of the four gradients (register budget)
-            rc = launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 1, 2>, grid, CS::bytes, stream, p, kXThreads16);
-            if (rc != SJVP_OK) return rc;
-            return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 2, 2>, grid, CS::bytes, stream, p, kXThreads16);
-        } else {
-            return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
-        }
-    } else {
-        // 32-wide pair for inputs of any alignment, same order
-        int rc = SJVP_OK;
-        if (parts & SJVP_BWD_ROW)
-            rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G>, BH * p.q_blocks, RowSmem<HD, HAS_G>::bytes, stream, p);
-        if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
-        const int col_grid = BH * p.k_blocks;
-        using SM = ColSmem<HD, HAS_DO, HAS_G>;
-        if constexpr (HD == 128) {
-            // two launches, each accumulating half of the head dimension (register budget)
-            rc = launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 0, 2>, col_grid, SM::bytes, stream, p);
-            if (rc != SJVP_OK) return rc;
-            return launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 2, 2>, col_grid, SM::bytes, stream, p);
-        } else {
-            return launch(bwd_col_kernel<T, HD, HAS_DO, HAS_G, true, true, 0, HD / 32>, col_grid, SM::bytes,
-                          stream, p);
-        }
-    }
-}
-
-template <typename T, int HD, bool DMA>
-int bwd_hd(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
-    if (has_do && has_g) return bwd_mode<T, HD, true, true, DMA>(p, BH, parts, stream);
-    if (has_g) return bwd_mode<T, HD, false, true, DMA>(p, BH, parts, stream);
-    return bwd_mode<T, HD, true, false, DMA>(p, BH, parts, stream);
-}
-
-template <typename T>
-int bwd_dtype(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
-    if (p.vec) {
-        if (p.D <= 32) return bwd_hd<T, 32, true>(p, BH, has_do, has_g, parts, stream);
-        if (p.D <= 64) return bwd_hd<T, 64, true>(p, BH, has_do, has_g, parts, stream);
-        return bwd_hd<T, 128, true>(p, BH, has_do, has_g, parts, stream);
-    }
-    if (p.D <= 32) return bwd_hd<T, 32, false>(p, BH, has_do, has_g, parts, stream);
-    if (p.D <= 64) return bwd_hd<T, 64, false>(p, BH, has_do, has_g, parts, stream);
-    return bwd_hd<T, 128, false>(p, BH, has_do, has_g, parts, stream);
+int bwd_select(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
+    if (!p.vec) return bwd_pair_any<T>(p, BH, has_do, has_g, parts, stream);
+    if (parts == SJVP_BWD_ALL && p.Lk <= kOwned16 && p.D <= 64) return bwd_fused<T>(p, BH, has_do, has_g, stream);
+    return bwd_pair_vec<T>(p, BH, has_do, has_g, parts, stream);
 }
 
 }  // namespace
@@ -197,7 +62,7 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     if (!q || !k || !v || !o || !lse || !strides) return SJVP_ERR_NULL;
     const bool jvp = tq || tk || tv || to || mu;
     if (jvp && (!tq || !tk || !tv || !to || !mu)) return SJVP_ERR_NULL;
-    int rc = check_common(B, H, Lq, Lk, D, dtype);
+    int rc = check_common(B, H, Lq, Lk, D, dtype, scale);
     if (rc != SJVP_OK) return rc;
 
     const void* ptrs[SJVP_F_COUNT] = {q, k, v, tq, tk, tv, o, to};
@@ -224,12 +89,14 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.D = D;
     p.Lr = round_up(Lq, 128);
     p.q_blocks = p.Lr / kOwned;  // covers every statistic row below Lr
-    p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+    p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
     const int grid = B * H * p.q_blocks;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == SJVP_BF16 ? fwd_dtype<Bf16>(p, grid, jvp, s) : fwd_dtype<Fp16>(p, grid, jvp, s);
+    // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
+    if (p.vec) return dtype == SJVP_BF16 ? fwd_vec<Bf16>(p, grid, jvp, s) : fwd_vec<Fp16>(p, grid, jvp, s);
+    return dtype == SJVP_BF16 ? fwd_any<Bf16>(p, grid, jvp, s) : fwd_any<Fp16>(p, grid, jvp, s);
 }
 
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype) {
@@ -260,7 +127,7 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
     const bool has_do = dO != nullptr, has_g = dTO != nullptr;
     if (!q || !k || !v || !o || !lse || !dq || !dk || !dv || !strides) return SJVP_ERR_NULL;
     if (has_g && (!tq || !tk || !tv || !to || !mu || !dtq || !dtk || !dtv)) return SJVP_ERR_NULL;
-    int rc = check_common(B, H, Lq, Lk, D, dtype);
+    int rc = check_common(B, H, Lq, Lk, D, dtype, scale);
     if (rc != SJVP_OK) return rc;
     if (!workspace || workspace_bytes < sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype) ||
         (reinterpret_cast<uintptr_t>(workspace) & 3u))
@@ -304,12 +171,12 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
     p.lse2 = static_cast<float*>(workspace);
     p.s4 = p.lse2 + (size_t)B * H * p.Lr;
     p.s7d = p.s4 + (size_t)B * H * p.Lr;
-    p.scale = scale > 0.f ? scale : 1.0f / sqrtf((float)D);
+    p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == SJVP_BF16 ? bwd_dtype<Bf16>(p, B * H, has_do, has_g, parts, s)
-                              : bwd_dtype<Fp16>(p, B * H, has_do, has_g, parts, s);
+    return dtype == SJVP_BF16 ? bwd_select<Bf16>(p, B * H, has_do, has_g, parts, s)
+                              : bwd_select<Fp16>(p, B * H, has_do, has_g, parts, s);
 }
 
 int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides, const float* cos,
@@ -356,9 +223,12 @@ int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* stride
     if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
 
     auto go = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)n), dim3(kRopeThreads), 0,
-                           static_cast<hipStream_t>(stream), p);
-        return hipGetLastError() == hipSuccess ? SJVP_OK : SJVP_ERR_LAUNCH;
+        RopeParams copy = p;
+        void* args[] = {&copy};
+        return hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3((unsigned)blocks, (unsigned)n),
+                               dim3(kRopeThreads), args, 0, static_cast<hipStream_t>(stream)) == hipSuccess
+                   ? SJVP_OK
+                   : SJVP_ERR_LAUNCH;
     };
     auto by_out = [&](auto in_tag) {
         using IN = decltype(in_tag);
@@ -382,11 +252,17 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
         case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
+        case SJVP_ERR_SCALE: return "scale must be finite and >= 0 (0 selects 1/sqrt(D))";
         case SJVP_ERR_ROTARY: return "sjvp_rope: n must be 1..4, rot_dim even and 2 <= rot_dim <= D, and bf16 / fp16 must not be mixed";
         default: return "unknown sjvp status";
     }
 }
 
 int sjvp_version(void) { return SJVP_VERSION; }
+
+#ifndef SJVP_BUILD_ID
+#define SJVP_BUILD_ID "SJVP_BUILD_ID=unknown"
+#endif
+const char* sjvp_build_id(void) { return SJVP_BUILD_ID; }
 
 }  // extern "C"

@@ -78,6 +78,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     const int b = bh / p.H, h = bh % p.H;
     const int key_slabs = (p.Lk + 31) >> 5;           // 32-key slabs that hold at least one key
     const bool wave_active = (wave >> 1) < key_slabs;  // waves of a partly filled slab all take part
+    // Keys beyond Lk are zero rows: their score is 0 and exp(-lse) overflows once every real score of
+    // a row is very negative, so their P is forced to zero (they would reach dQ, dQ_dot of valid
+    // queries through the bounce tile as 0 * inf otherwise).  Wave-uniform flag, per-lane predicate.
+    const bool ragged_keys = wave * 16 + 16 > p.Lk;
+    const bool key_padded = wave * 16 + n >= p.Lk;
 
     // own rows first (they land first), then the ring
     {
@@ -212,7 +217,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
+                float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
+                if (ragged_keys && key_padded) pj = 0.f;
                 s[t][j] = pj;
                 if constexpr (HAS_G) {
                     const float nn = fmaf(ts[t][j], p.scale, -mu4[j]);

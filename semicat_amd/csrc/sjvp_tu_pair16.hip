@@ -1,0 +1,46 @@
+// Translation unit: 16-wide row-owned + column-owned backward pair for one element type (SJVP_T).
+#include "sjvp_bwd16x.hpp"
+#include "sjvp_launch.hpp"
+
+namespace sjvp {
+namespace {
+
+template <typename T, int HD, bool HAS_DO, bool HAS_G>
+int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
+    // the row-owned kernel first (besides dQ, dQ_dot it leaves the row sums in the workspace), then
+    // the column-owned one; workgroups of four waves own 64 positions
+    constexpr int XR = HD == 128 ? 2 : 3;  // ring depth
+    int rc = SJVP_OK;
+    if (parts & SJVP_BWD_ROW)
+        rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, (HD == 128 ? 2 : 3)>,
+                    BH * (p.Lr / kXOwned16), Row16Smem<HD, XR, HAS_G>::bytes, stream, p, kXThreads16);
+    if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
+    const int grid = BH * ((p.Lk + kXOwned16 - 1) / kXOwned16);
+    using CS = Col16Smem<HD, XR, HAS_DO, HAS_G>;
+    if constexpr (HD == 128) {
+        // two launches, each accumulating two of the four gradients (register budget)
+        rc = launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 1, 2>, grid, CS::bytes, stream, p, kXThreads16);
+        if (rc != SJVP_OK) return rc;
+        return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 2, 2>, grid, CS::bytes, stream, p, kXThreads16);
+    } else {
+        return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
+    }
+}
+
+template <typename T, int HD>
+int pair_hd(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
+    if (has_do && has_g) return pair_mode<T, HD, true, true>(p, BH, parts, stream);
+    if (has_g) return pair_mode<T, HD, false, true>(p, BH, parts, stream);
+    return pair_mode<T, HD, true, false>(p, BH, parts, stream);
+}
+
+}  // namespace
+
+template <>
+int bwd_pair_vec<SJVP_T>(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
+    if (p.D <= 32) return pair_hd<SJVP_T, 32>(p, BH, has_do, has_g, parts, stream);
+    if (p.D <= 64) return pair_hd<SJVP_T, 64>(p, BH, has_do, has_g, parts, stream);
+    return pair_hd<SJVP_T, 128>(p, BH, has_do, has_g, parts, stream);
+}
+
+}  // namespace sjvp

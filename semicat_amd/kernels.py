@@ -23,6 +23,17 @@ from . import _lib
 _DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16}
 
 
+def _scale_arg(scale: Optional[float]) -> float:
+    """The C ABI's spelling of the softmax scale: 0.0 selects 1/sqrt(D), which is what ``None`` means
+    in the reference wrappers (ryu_triton.py:324-325); anything else must be a positive finite number."""
+    if scale is None:
+        return 0.0
+    scale = float(scale)
+    if not (scale > 0.0) or math.isinf(scale):
+        raise ValueError(f"scale must be a positive finite number or None, got {scale}")
+    return scale
+
+
 def stat_rows(L: int) -> int:
     """Length of the row-statistic buffers: L rounded up to 128 (ryu_triton.py:351)."""
     return ((L + 127) // 128) * 128
@@ -117,7 +128,7 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=
         stream = torch.cuda.current_stream().cuda_stream
         args = (_ptr(q), _ptr(k), _ptr(v), _ptr(tq), _ptr(tk), _ptr(tv), _ptr(o), _ptr(to),
                 _ptr(lse), _ptr(mu), _ptr(li), B, H, Lq, Lk, D, _strides((q, k, v, tq, tk, tv, o, to)),
-                float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+                _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
         if _plan:
             return _Launch(lib.sjvp_fwd, args, (q, k, v, tq, tk, tv, o, to, lse, mu, li)), (o, to, lse, mu, li)
         rc = lib.sjvp_fwd(*args)
@@ -148,7 +159,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.sjvp_fwd(_ptr(q), _ptr(k), _ptr(v), None, None, None, _ptr(o), None, _ptr(lse), None,
                           None, B, H, Lq, Lk, D, _strides((q, k, v, None, None, None, o, None)),
-                          float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+                          _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
     _lib.check(rc)
     return o, lse
 
@@ -225,7 +236,7 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         stream = torch.cuda.current_stream().cuda_stream
         args = (int(parts), *(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
                 *(_ptr(t) for t in tensors[10:]), _ptr(workspace), nbytes, B, H, Lq, Lk, D,
-                _strides(tensors), float(scale) if scale else 0.0, dtype_tag, ctypes.c_void_p(stream))
+                _strides(tensors), _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
         if _plan:
             return (_Launch(lib.sjvp_bwd_parts, args, tensors + (lse, mu, workspace)),
                     (dq, dk, dv, dtq, dtk, dtv))
@@ -267,19 +278,27 @@ def flash_jvp_backward(dto, q, k, v, o, tq, tk, tv, lse, mu, li, dq, dk, dv, dtq
                        softmax_scale: Optional[float] = None, *, to=None) -> None:
     """Signature of ``flash_jvp_backward._flash_attn_backward`` (flash_jvp_backward.py:2293-2312):
     every tensor is [B,S,H,D]; fills the six gradients in place for the cotangent ``dto`` on the
-    tangent output.  ``o`` must be the primal output and ``to`` the tangent output of the forward:
-    the row sums are taken from them instead of being recomputed with five contractions.  ``li`` is
-    accepted and ignored (it is not needed mathematically)."""
-    if to is None:
-        raise ValueError("flash_jvp_backward needs the forward's tangent output as keyword `to` "
-                         "(and its primal output as `o`)")
+    tangent output.  ``li`` is accepted and ignored (it is not needed mathematically).
+
+    The reference never reads its ``o`` argument (its call site passes the tangent output there,
+    functional.py:131-149) and recomputes the row sums ``rowsum(dto*O)``, ``rowsum(dto*TO)`` with five
+    contractions.  Here they are formed from ``O`` and ``TO`` directly: called with the reference's 17
+    positional arguments, ``o`` is ignored as well and both are recomputed with one fused forward
+    launch; a caller that still holds them passes the primal output as ``o`` and the tangent output
+    as keyword ``to`` and saves that launch."""
     for tan, tan_grad in zip((tq, tk, tv), (dtq, dtk, dtv)):  # flash_jvp_backward.py:2419-2428
         for i in range(tan.dim()):
             if tan.shape[i] != tan_grad.shape[i]:
                 raise ValueError(f"Tangent and tangent gradient have different shapes: "
                                  f"{tan.shape} != {tan_grad.shape}")
-    attention_jvp_backward(_bshd(q), _bshd(k), _bshd(v), _bshd(tq), _bshd(tk), _bshd(tv), _bshd(o),
-                           _bshd(to), lse, mu, dO=None, dTO=_bshd(dto), scale=softmax_scale,
+    scale = softmax_scale or None  # flash_jvp_backward.py:2323: a zero scale means the default
+    if to is None:
+        o_bh, to_bh, _, _, _ = attention_jvp_forward(_bshd(q), _bshd(k), _bshd(v), _bshd(tq), _bshd(tk),
+                                                     _bshd(tv), scale=scale, with_li=False)
+    else:
+        o_bh, to_bh = _bshd(o), _bshd(to)
+    attention_jvp_backward(_bshd(q), _bshd(k), _bshd(v), _bshd(tq), _bshd(tk), _bshd(tv), o_bh,
+                           to_bh, lse, mu, dO=None, dTO=_bshd(dto), scale=scale,
                            grads=tuple(_bshd(g) for g in (dq, dk, dv, dtq, dtk, dtv)))
 
 
@@ -291,12 +310,8 @@ def flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal: bool
     if bias is not None or causal:
         raise NotImplementedError("the attention-JVP path is non-causal and bias-free")
     attention_jvp_backward(_bshd(q), _bshd(k), _bshd(v), None, None, None, _bshd(o), None, lse, None,
-                           dO=_bshd(do), dTO=None, scale=softmax_scale,
+                           dO=_bshd(do), dTO=None, scale=softmax_scale or None,
                            grads=(_bshd(dq), _bshd(dk), _bshd(dv), None, None, None))
-
-
-def default_scale(D: int) -> float:
-    return 1.0 / math.sqrt(D)
 
 
 _ROPE_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16, torch.float32: _lib.SJVP_FP32}

@@ -178,6 +178,53 @@ def test_self_distillation_step_through_the_op_gpu():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("sd_prop", [0.25, 1.0])
+def test_full_size_step_gpu(sd_prop):
+    """The training configuration at its real size (configs/model/text8_dit_lg.yaml:8-15,
+    configs/experiment/lm1b_dit.yaml:15-23): 12 blocks, d_model 768, 12 heads of 64, cond_dim 128,
+    sequence 128, vocabulary 30522, batch 64, bf16 autocast, random token ids.  The first
+    int(sd_prop * 64) samples take the self-distillation loss through the HIP attention-JVP and
+    rotary kernels, the others the cross-entropy loss (semicat.py:186-191; the reference default is
+    sd_prop = 0.25, and sd_prop = 1 makes every attention call the benchmark's shape).  Losses finite
+    and equal to the same network with eager math attention and the PyTorch rotary."""
+    from semicat_amd import _lib
+    _lib.load()
+    B, S, V = 64, 128, 30522
+    print(f"[full-size step] sd_prop={sd_prop}", flush=True)
+    net = make_net(vocab=V, hidden=768, heads=12, blocks=12, length=S, cond=128, rotary="hip").cuda()
+    torch.manual_seed(5)
+    x1 = torch.randint(0, V, (B, S), device="cuda")
+    x0 = torch.randn(B, S, V, device="cuda")
+    t = torch.rand(B, device="cuda")
+    s = torch.rand(B, device="cuda") * t
+    split = int(sd_prop * B)
+    watched = ("blocks.0.attn_qkv.weight", "blocks.11.attn_qkv.weight", "blocks.5.mlp.0.weight",
+               "vocab_embed.seq.weight")
+    results = []
+    for override, rotary in ((None, "hip"), (math_attention, "torch")):
+        net.attention_override, net.rotary = override, rotary
+        net.zero_grad(set_to_none=True)
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            sd = ts.lag_self_distillation_loss(net, x0[:split], x1[:split], t=t[:split], s=s[:split])
+            vf = ts.vfm_loss(net, x0[split:], x1[split:], t=t[split:]) if split < B else None
+        (sd if vf is None else vf + sd).backward()
+        params = dict(net.named_parameters())
+        results.append((sd.item(), None if vf is None else vf.item(),
+                        {n: params[n].grad.detach().float().clone() for n in watched}))
+        torch.cuda.synchronize()
+    (sd_a, vf_a, g_a), (sd_b, vf_b, g_b) = results
+    print(f"[full-size step] sd {sd_a:.6g} vs {sd_b:.6g}; vfm {vf_a} vs {vf_b}", flush=True)
+    assert math.isfinite(sd_a) and abs(sd_a - sd_b) <= 3e-2 * abs(sd_b), (sd_a, sd_b)
+    if vf_a is not None:
+        assert math.isfinite(vf_a) and abs(vf_a - vf_b) <= 3e-2 * abs(vf_b), (vf_a, vf_b)
+    for n in watched:
+        assert torch.isfinite(g_a[n]).all(), n
+        err = ((g_a[n] - g_b[n]).norm() / g_b[n].norm()).item()
+        print(f"[full-size step] grad {n}: rel err {err:.3e}", flush=True)
+        assert err <= 1e-1, (n, err)
+
+
+@pytest.mark.gpu
 def test_plain_attention_modes_agree_gpu():
     from semicat_amd import _lib
     _lib.load()

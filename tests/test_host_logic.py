@@ -157,8 +157,9 @@ def test_library_exports_every_declared_symbol(repo_root):
     header = open(os.path.join(repo_root, "include", "sjvp.h")).read()
     declared = set(re.findall(r"\b(sjvp_[a-z_]+)\s*\(", header))
     assert declared == set(_lib.EXPORTS)
-    if not os.path.exists(build.LIB_PATH):
+    if build.is_stale():
         build.build()
+    assert build.built_id() == build.source_id()
     lib = ctypes.CDLL(build.LIB_PATH)
     for name in declared:
         assert hasattr(lib, name), name
@@ -166,7 +167,7 @@ def test_library_exports_every_declared_symbol(repo_root):
     assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
     assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4
     assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4
-    for code in range(0, -10, -1):
+    for code in range(0, -11, -1):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
@@ -185,6 +186,14 @@ def test_c_abi_argument_errors_are_reported_before_any_launch():
     assert f(dtype=7) == _lib.SJVP_ERR_DTYPE
     assert f(B=0) == _lib.SJVP_ERR_SHAPE
     assert f(Lq=0) == _lib.SJVP_ERR_SHAPE
+    # scale: 0 selects 1/sqrt(D); negative, infinite and NaN are refused
+    for bad in (-1.0, float("inf"), float("nan")):
+        assert L.sjvp_fwd(one, one, one, one, one, one, one, one, one, one, one, 1, 1, 8, 8, 64, strides,
+                          bad, 0, None) == _lib.SJVP_ERR_SCALE
+    for bad in (0.0, -0.5, float("inf")):
+        with pytest.raises(ValueError):
+            kernels._scale_arg(bad)
+    assert kernels._scale_arg(None) == 0.0 and kernels._scale_arg(0.125) == 0.125
     assert L.sjvp_fwd(None, one, one, one, one, one, one, one, one, one, one, 1, 1, 8, 8, 64, strides,
                       0.0, 0, None) == _lib.SJVP_ERR_NULL
     # tangent inputs must come all together
