@@ -23,8 +23,9 @@
  *   - scale == 0 selects the default 1/sqrt(D) (ryu_triton.py:324-325); a negative or non-finite
  *     scale is an error.
  *   - The caller owns every buffer, including the workspace; the library allocates no device
- *     memory, keeps no pointer after returning, has no mutable global state, enqueues on the given
- *     hipStream_t (passed as void*) of the CURRENT device and returns without synchronising.
+ *     memory, keeps no pointer after returning, has no mutable global state (except the per-device
+ *     address of sjvp_bwd_noalloc()'s static scratch), enqueues on the given hipStream_t (passed as
+ *     void*) of the CURRENT device and returns without synchronising.
  *   - Every function returns SJVP_OK (0) or a negative error code; nothing aborts or throws.
  *     Argument errors are detected before anything is launched.
  *   - Results are deterministic: no atomics are used.
@@ -54,7 +55,8 @@ enum sjvp_status {
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
     SJVP_ERR_PARTS = -8,     /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
     SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16 */
-    SJVP_ERR_SCALE = -10     /* scale negative, infinite or NaN (0 selects the default)      */
+    SJVP_ERR_SCALE = -10,    /* scale negative, infinite or NaN (0 selects the default)      */
+    SJVP_ERR_SCRATCH = -11   /* sjvp_bwd_noalloc: problem beyond SJVP_NOALLOC_MAX_ROWS, or no static scratch on this device */
 };
 
 /* Indices into the stride tables: strides[3*i + {0,1,2}] = (batch, head, sequence) strides in
@@ -107,6 +109,28 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
                    void* dtq, void* dtk, void* dtv, void* workspace, size_t workspace_bytes, int B,
                    int H, int Lq, int Lk, int D, const int64_t* strides /* [SJVP_B_COUNT*3] */,
                    float scale, int dtype, void* stream);
+
+/*
+ * sjvp_bwd() with the workspace taken from a static device array inside the library instead of a
+ * caller buffer.  It has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  The call allocates and frees nothing (neither does the rest of this library).
+ *   - Limit: B * H * ceil(Lq/128)*128 <= SJVP_NOALLOC_MAX_ROWS (1 Mi statistic rows, 12 MiB of
+ *     device memory that every GPU the library runs on holds until the process ends); larger
+ *     problems return SJVP_ERR_SCRATCH and must use sjvp_bwd().
+ *   - Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams,
+ *     two threads) race on it.  Calls on one stream are ordered and safe; nothing has to be cleared
+ *     between calls (each launch pair writes every row it later reads).
+ *   - The array's address is looked up on the first call on each device (no allocation); make that
+ *     first call outside a graph capture.
+ * Same results as sjvp_bwd(), bit for bit.
+ */
+#define SJVP_NOALLOC_MAX_ROWS (1 << 20)
+int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                     const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+                     const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq,
+                     void* dtk, void* dtv, int B, int H, int Lq, int Lk, int D,
+                     const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
 
 /* Bytes of caller-provided device scratch sjvp_bwd needs: lse in log2 units and the row sums sum_4
  * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,

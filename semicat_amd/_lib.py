@@ -22,6 +22,8 @@ SJVP_ERR_COTANGENT = -7
 SJVP_ERR_PARTS = -8
 SJVP_ERR_ROTARY = -9
 SJVP_ERR_SCALE = -10
+SJVP_ERR_SCRATCH = -11
+SJVP_NOALLOC_MAX_ROWS = 1 << 20
 
 SJVP_BWD_ROW = 1
 SJVP_BWD_COL = 2
@@ -31,7 +33,7 @@ F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
 B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
-EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_workspace_bytes", "sjvp_rope",
+EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_noalloc", "sjvp_bwd_workspace_bytes", "sjvp_rope",
            "sjvp_strerror", "sjvp_version", "sjvp_build_id")
 
 _lock = threading.Lock()
@@ -63,6 +65,9 @@ def load() -> ctypes.CDLL:
             lib.sjvp_bwd.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [vp, ctypes.c_size_t] + [i] * 5 +
                                      [i64p, ctypes.c_float, i, vp])
             lib.sjvp_bwd.restype = i
+            lib.sjvp_bwd_noalloc.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [i] * 5 +
+                                             [i64p, ctypes.c_float, i, vp])
+            lib.sjvp_bwd_noalloc.restype = i
             lib.sjvp_bwd_parts.argtypes = [i] + lib.sjvp_bwd.argtypes
             lib.sjvp_bwd_parts.restype = i
             lib.sjvp_bwd_workspace_bytes.argtypes = [i] * 6

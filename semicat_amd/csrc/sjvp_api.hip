@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
+#include <mutex>
+
 #include "sjvp_launch.hpp"
 #include "sjvp_rope.hpp"
 #include "sjvp_w16.hpp"
@@ -50,6 +52,96 @@ int bwd_select(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, h
     if (!p.vec) return bwd_pair_any<T>(p, BH, has_do, has_g, parts, stream);
     if (parts == SJVP_BWD_ALL && p.Lk <= kOwned16 && p.D <= 64) return bwd_fused<T>(p, BH, has_do, has_g, stream);
     return bwd_pair_vec<T>(p, BH, has_do, has_g, parts, stream);
+}
+
+// The backward's tensors as they arrive through the C ABI.
+struct BwdTensors {
+    const void *q, *k, *v, *tq, *tk, *tv, *o, *to, *dO, *dTO;
+    const float *lse, *mu;
+    void *dq, *dk, *dv, *dtq, *dtk, *dtv;
+};
+
+int check_bwd(int parts, const BwdTensors& t, int B, int H, int Lq, int Lk, int D, const int64_t* strides,
+              float scale, int dtype) {
+    if (parts < SJVP_BWD_ROW || parts > SJVP_BWD_ALL) return SJVP_ERR_PARTS;
+    if (!t.dO && !t.dTO) return SJVP_ERR_COTANGENT;
+    if (!t.q || !t.k || !t.v || !t.o || !t.lse || !t.dq || !t.dk || !t.dv || !strides) return SJVP_ERR_NULL;
+    if (t.dTO && (!t.tq || !t.tk || !t.tv || !t.to || !t.mu || !t.dtq || !t.dtk || !t.dtv)) return SJVP_ERR_NULL;
+    return check_common(B, H, Lq, Lk, D, dtype, scale);
+}
+
+// Launches of the backward on a validated problem; `ws` holds 3 * B * H * Lr floats.
+int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int Lk, int D,
+            const int64_t* strides, float scale, int dtype, void* stream) {
+    const bool has_do = t.dO != nullptr, has_g = t.dTO != nullptr;
+    const void* ptrs[SJVP_B_COUNT] = {t.q, t.k, t.v, has_g ? t.tq : nullptr, has_g ? t.tk : nullptr,
+                                      has_g ? t.tv : nullptr, t.o, has_g ? t.to : nullptr, t.dO, t.dTO,
+                                      t.dq, t.dk, t.dv, has_g ? t.dtq : nullptr, has_g ? t.dtk : nullptr,
+                                      has_g ? t.dtv : nullptr};
+    VecCheck vc;
+    for (int i = 0; i < SJVP_B_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
+
+    BwdParams p{};
+    p.q = view(t.q, strides + 3 * SJVP_B_Q);
+    p.k = view(t.k, strides + 3 * SJVP_B_K);
+    p.v = view(t.v, strides + 3 * SJVP_B_V);
+    p.o = view(t.o, strides + 3 * SJVP_B_O);
+    if (has_do) p.dO = view(t.dO, strides + 3 * SJVP_B_DO);
+    p.dq = out_view(t.dq, strides + 3 * SJVP_B_DQ);
+    p.dk = out_view(t.dk, strides + 3 * SJVP_B_DK);
+    p.dv = out_view(t.dv, strides + 3 * SJVP_B_DV);
+    if (has_g) {
+        p.tq = view(t.tq, strides + 3 * SJVP_B_TQ);
+        p.tk = view(t.tk, strides + 3 * SJVP_B_TK);
+        p.tv = view(t.tv, strides + 3 * SJVP_B_TV);
+        p.to = view(t.to, strides + 3 * SJVP_B_TO);
+        p.dTO = view(t.dTO, strides + 3 * SJVP_B_DTO);
+        p.dtq = out_view(t.dtq, strides + 3 * SJVP_B_DTQ);
+        p.dtk = out_view(t.dtk, strides + 3 * SJVP_B_DTK);
+        p.dtv = out_view(t.dtv, strides + 3 * SJVP_B_DTV);
+    }
+    p.lse = t.lse;
+    p.mu = t.mu;
+    p.H = H;
+    p.Lq = Lq;
+    p.Lk = Lk;
+    p.D = D;
+    p.Lr = round_up(Lq, 128);
+    p.q_blocks = p.Lr / kOwned;
+    p.k_blocks = round_up(Lk, kOwned) / kOwned;
+    p.lse2 = ws;
+    p.s4 = p.lse2 + (size_t)B * H * p.Lr;
+    p.s7d = p.s4 + (size_t)B * H * p.Lr;
+    p.scale = resolve_scale(scale, D);
+    p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == SJVP_BF16 ? bwd_select<Bf16>(p, B * H, has_do, has_g, parts, s)
+                              : bwd_select<Fp16>(p, B * H, has_do, has_g, parts, s);
+}
+
+// Scratch of sjvp_bwd_noalloc(): the backward's workspace (lse in log2 units and the two row sums,
+// 3 floats per statistic row) for up to SJVP_NOALLOC_MAX_ROWS rows, resident in every GPU the library
+// runs on from the moment its code is loaded until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress(); its device address differs from GPU to GPU and is
+// looked up once per device, with that device current.
+static __device__ __align__(256) __attribute__((used)) float scratch[3 * (size_t)SJVP_NOALLOC_MAX_ROWS];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SJVP_ERR_SCRATCH;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return SJVP_ERR_SCRATCH;
+        g_scratch_ptr[dev] = static_cast<float*>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return SJVP_OK;
 }
 
 }  // namespace
@@ -122,61 +214,28 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
                    void* dtq, void* dtk, void* dtv, void* workspace, size_t workspace_bytes, int B,
                    int H, int Lq, int Lk, int D, const int64_t* strides, float scale, int dtype,
                    void* stream) {
-    if (parts < SJVP_BWD_ROW || parts > SJVP_BWD_ALL) return SJVP_ERR_PARTS;
-    if (!dO && !dTO) return SJVP_ERR_COTANGENT;
-    const bool has_do = dO != nullptr, has_g = dTO != nullptr;
-    if (!q || !k || !v || !o || !lse || !dq || !dk || !dv || !strides) return SJVP_ERR_NULL;
-    if (has_g && (!tq || !tk || !tv || !to || !mu || !dtq || !dtk || !dtv)) return SJVP_ERR_NULL;
-    int rc = check_common(B, H, Lq, Lk, D, dtype, scale);
+    const BwdTensors t{q, k, v, tq, tk, tv, o, to, dO, dTO, lse, mu, dq, dk, dv, dtq, dtk, dtv};
+    int rc = check_bwd(parts, t, B, H, Lq, Lk, D, strides, scale, dtype);
     if (rc != SJVP_OK) return rc;
     if (!workspace || workspace_bytes < sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype) ||
         (reinterpret_cast<uintptr_t>(workspace) & 3u))
         return SJVP_ERR_WORKSPACE;
+    return run_bwd(parts, t, static_cast<float*>(workspace), B, H, Lq, Lk, D, strides, scale, dtype, stream);
+}
 
-    const void* ptrs[SJVP_B_COUNT] = {q, k, v, has_g ? tq : nullptr, has_g ? tk : nullptr,
-                                      has_g ? tv : nullptr, o, has_g ? to : nullptr, dO, dTO, dq, dk,
-                                      dv, has_g ? dtq : nullptr, has_g ? dtk : nullptr,
-                                      has_g ? dtv : nullptr};
-    VecCheck vc;
-    for (int i = 0; i < SJVP_B_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
-
-    BwdParams p{};
-    p.q = view(q, strides + 3 * SJVP_B_Q);
-    p.k = view(k, strides + 3 * SJVP_B_K);
-    p.v = view(v, strides + 3 * SJVP_B_V);
-    p.o = view(o, strides + 3 * SJVP_B_O);
-    if (has_do) p.dO = view(dO, strides + 3 * SJVP_B_DO);
-    p.dq = out_view(dq, strides + 3 * SJVP_B_DQ);
-    p.dk = out_view(dk, strides + 3 * SJVP_B_DK);
-    p.dv = out_view(dv, strides + 3 * SJVP_B_DV);
-    if (has_g) {
-        p.tq = view(tq, strides + 3 * SJVP_B_TQ);
-        p.tk = view(tk, strides + 3 * SJVP_B_TK);
-        p.tv = view(tv, strides + 3 * SJVP_B_TV);
-        p.to = view(to, strides + 3 * SJVP_B_TO);
-        p.dTO = view(dTO, strides + 3 * SJVP_B_DTO);
-        p.dtq = out_view(dtq, strides + 3 * SJVP_B_DTQ);
-        p.dtk = out_view(dtk, strides + 3 * SJVP_B_DTK);
-        p.dtv = out_view(dtv, strides + 3 * SJVP_B_DTV);
-    }
-    p.lse = lse;
-    p.mu = mu;
-    p.H = H;
-    p.Lq = Lq;
-    p.Lk = Lk;
-    p.D = D;
-    p.Lr = round_up(Lq, 128);
-    p.q_blocks = p.Lr / kOwned;
-    p.k_blocks = round_up(Lk, kOwned) / kOwned;
-    p.lse2 = static_cast<float*>(workspace);
-    p.s4 = p.lse2 + (size_t)B * H * p.Lr;
-    p.s7d = p.s4 + (size_t)B * H * p.Lr;
-    p.scale = resolve_scale(scale, D);
-    p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
-
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == SJVP_BF16 ? bwd_select<Bf16>(p, B * H, has_do, has_g, parts, s)
-                              : bwd_select<Fp16>(p, B * H, has_do, has_g, parts, s);
+int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                     const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+                     const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq,
+                     void* dtk, void* dtv, int B, int H, int Lq, int Lk, int D, const int64_t* strides,
+                     float scale, int dtype, void* stream) {
+    const BwdTensors t{q, k, v, tq, tk, tv, o, to, dO, dTO, lse, mu, dq, dk, dv, dtq, dtk, dtv};
+    int rc = check_bwd(SJVP_BWD_ALL, t, B, H, Lq, Lk, D, strides, scale, dtype);
+    if (rc != SJVP_OK) return rc;
+    if ((int64_t)B * H * round_up(Lq, 128) > (int64_t)SJVP_NOALLOC_MAX_ROWS) return SJVP_ERR_SCRATCH;
+    float* ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc != SJVP_OK) return rc;
+    return run_bwd(SJVP_BWD_ALL, t, ws, B, H, Lq, Lk, D, strides, scale, dtype, stream);
 }
 
 int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides, const float* cos,
@@ -253,6 +312,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
         case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
         case SJVP_ERR_SCALE: return "scale must be finite and >= 0 (0 selects 1/sqrt(D))";
+        case SJVP_ERR_SCRATCH: return "sjvp_bwd_noalloc: B * H * ceil(Lq/128)*128 exceeds SJVP_NOALLOC_MAX_ROWS, or the static scratch could not be located on this device";
         case SJVP_ERR_ROTARY: return "sjvp_rope: n must be 1..4, rot_dim even and 2 <= rot_dim <= D, and bf16 / fp16 must not be mixed";
         default: return "unknown sjvp status";
     }

@@ -166,13 +166,17 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
 
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
                            scale: Optional[float] = None, grads=None, workspace=None,
-                           parts: int = _lib.SJVP_BWD_ALL, _plan: bool = False):
+                           parts: int = _lib.SJVP_BWD_ALL, static_scratch: bool = False,
+                           _plan: bool = False):
     """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
     Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
     tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
     (the tangent three may be None without dTO); ``workspace`` a uint8 device buffer of at least
     ``sjvp_bwd_workspace_bytes`` bytes (allocated here otherwise).  ``parts`` selects the launches
-    (profiling only: SJVP_BWD_COL alone needs the workspace an earlier SJVP_BWD_ROW call filled)."""
+    (profiling only: SJVP_BWD_COL alone needs the workspace an earlier SJVP_BWD_ROW call filled).
+    ``static_scratch=True`` takes the ``sjvp_bwd_noalloc`` entry point instead: the workspace is a
+    static device array of the library, so with ``grads`` supplied the call allocates nothing; it
+    serves up to ``SJVP_NOALLOC_MAX_ROWS`` statistic rows and calls overlapping on one GPU race."""
     dtype_tag = _require_gpu(q)
     if dO is None and dTO is None:
         raise ValueError("attention_jvp_backward needs a cotangent on o, on to, or on both")
@@ -226,12 +230,22 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
     if B * H * Lq == 0 and not _plan:
         return dq, dk, dv, dtq, dtk, dtv
     lib = _lib.load()
+    tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
+    if static_scratch:
+        if workspace is not None or parts != _lib.SJVP_BWD_ALL or _plan:
+            raise ValueError("static_scratch excludes workspace, parts and planned launches")
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = lib.sjvp_bwd_noalloc(*(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
+                                      *(_ptr(t) for t in tensors[10:]), B, H, Lq, Lk, D, _strides(tensors),
+                                      _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
+        _lib.check(rc)
+        return dq, dk, dv, dtq, dtk, dtv
     nbytes = lib.sjvp_bwd_workspace_bytes(B, H, Lq, Lk, D, dtype_tag)
     if workspace is None:
         workspace = torch.empty((nbytes,), device=dev, dtype=torch.uint8)
     elif workspace.dtype != torch.uint8 or workspace.numel() < nbytes or workspace.device != dev:
         raise AssertionError(f"workspace must be a uint8 tensor of >= {nbytes} bytes on {dev}")
-    tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
         args = (int(parts), *(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),

@@ -167,7 +167,7 @@ def test_library_exports_every_declared_symbol(repo_root):
     assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
     assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4
     assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4
-    for code in range(0, -11, -1):
+    for code in range(0, -12, -1):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
@@ -205,6 +205,10 @@ def test_c_abi_argument_errors_are_reported_before_any_launch():
     assert b(None, None, one, 1 << 20) == _lib.SJVP_ERR_COTANGENT
     assert b(one, one, None, 1 << 20) == _lib.SJVP_ERR_WORKSPACE
     assert b(one, one, one, 8) == _lib.SJVP_ERR_WORKSPACE
+    # the no-allocation backward refuses what its static scratch cannot hold, before any HIP call
+    assert L.sjvp_bwd_noalloc(*([one] * 18), 64, 16, 1025, 128, 64, strides, 0.0, 0, None) == _lib.SJVP_ERR_SCRATCH
+    assert L.sjvp_bwd_noalloc(*([one] * 8), None, None, *([one] * 8), 1, 1, 8, 8, 64, strides, 0.0, 0,
+                              None) == _lib.SJVP_ERR_COTANGENT
     with pytest.raises(_lib.SjvpError):
         _lib.check(_lib.SJVP_ERR_HEAD_DIM)
     # sjvp_rope
