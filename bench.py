@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention-JVP forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--graph] [--no-cpu-baseline] [--no-cold] [--no-hardware] [--calib-copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--graph] [--no-cpu-baseline] [--no-cold] [--no-hardware] [--no-autograd] [--calib-copy]
 
 A step is one pass of the hot path over one batch: the fused forward (O, TO, lse, mu) followed by
 the backward for cotangents on both O and TO (six gradients), on the LM1B-shaped configuration
@@ -31,12 +31,37 @@ PRIMAL_SCALE, TANGENT_SCALE, SEED = 0.5, 0.1, 0
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 NAMES = ("q", "k", "v", "tq", "tk", "tv", "dO", "dTO")
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, scaled by the copy
-# kernel of --calib-copy: one FETCH_SIZE unit is 2 KiB, one WRITE_SIZE unit 1 KiB there).
-MEASURED_TRAFFIC_BYTES = {
-    "fwd16_kernel": (2 * 36937.5 + 25344.4) * 1024,
-    "bwd_fused16_kernel": (2 * 61934.8 + 73985.3) * 1024,
-}
+# HBM bytes per launch come from rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE per
+# dispatch, scaled by what the same counters read on the copy kernel of --calib-copy); the summary of
+# those runs keeps them as "traffic: <kernel> fetch <units> x <KiB per unit> write <units> x <KiB per
+# unit> commit <hash>" lines, which is where roofline.traffic is read from.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "kernels_config2_bf16.md")
+
+
+def measured_traffic(kernel: str):
+    """(HBM bytes per launch, source) for a kernel from the committed profiler summary, or (None, None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                w = line.split()
+                if len(w) >= 12 and w[0] == "traffic:" and w[1] == kernel:
+                    fetch, fetch_kib, write, write_kib = float(w[3]), float(w[5]), float(w[7]), float(w[9])
+                    src = f"profiles/{os.path.basename(TRAFFIC_FILE)} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit {w[11]})"
+                    return (fetch * fetch_kib + write * write_kib) * 1024.0, src
+    except OSError:
+        pass
+    return None, None
+
+
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def step_flops(b=B, h=H, l=L, d=D) -> float:
@@ -57,32 +82,66 @@ def make_inputs(device, b=B):
     return out
 
 
-def cpu_baseline(seconds: float = 12.0):
-    """The reference's CPU math path (torch.func.jvp over eager softmax(QK^T s)V, then autograd for the
-    six gradients; oracle.attention_jvp_autograd in fp32) on a bounded sample of the same workload:
-    the first 8 of the 64 batches, bf16 inputs up-cast to fp32, all host threads torch uses."""
-    from oracle import attn_jvp_oracle as orc
-    sample_b = 8
-    x = make_inputs("cpu", b=sample_b)
-    args = [x[n] for n in NAMES]
-    run = lambda: orc.attention_jvp_autograd(*args, dtype=torch.float32)
+def _time_cpu(run, seconds: float, max_runs: int = 50):
+    run()
     run()
     times = []
     t_end = time.perf_counter() + seconds
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < max_runs):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     times.sort()
-    med = times[len(times) // 2]
+    return times[len(times) // 2], len(times)
+
+
+def cpu_baseline(seconds: float = 10.0):
+    """The reference's CPU math path (torch.func.jvp over eager softmax(QK^T s)V, then autograd for the
+    six gradients; oracle.attention_jvp_autograd in fp32) on all host threads torch uses, 2 warm-ups and
+    the median of at least 5 runs each: on a bounded sample of the metric's workload (the first 8 of the
+    64 batches of config 2, bf16 inputs up-cast to fp32), and on config 1 (B=2, H=4, L=256, D=64, fp32
+    N(0,1) inputs, seed 0) in full."""
+    from oracle import attn_jvp_oracle as orc
+    sample_b = 8
+    x = make_inputs("cpu", b=sample_b)
+    args = [x[n] for n in NAMES]
+    med, n_runs = _time_cpu(lambda: orc.attention_jvp_autograd(*args, dtype=torch.float32), seconds)
+    x1 = orc.make_inputs(2, 4, 256, 256, 64, seed=0, dtype=torch.float32)
+    args1 = [x1[n] for n in orc.TENSOR_ORDER]
+    med1, n1 = _time_cpu(lambda: orc.attention_jvp_autograd(*args1, dtype=torch.float32), seconds / 2)
     return {
         "value": step_flops(b=sample_b) / med / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
+        "cpu_model": cpu_model(),
         "kind": "port",
         "sample": f"B={sample_b} of 64 (H=12,L=128,D=64), fp32 eager torch.func.jvp + autograd.grad, "
-                  f"median of {len(times)} runs, {med * 1e3:.1f} ms each",
+                  f"median of {n_runs} runs, {med * 1e3:.1f} ms each",
+        "config1": {"value": step_flops(2, 4, 256, 64) / med1 / 1e12, "unit": "TFLOP/s",
+                    "sample": f"config 1 in full (B=2,H=4,L=256,D=64, fp32, seed 0), median of {n1} runs, "
+                              f"{med1 * 1e3:.1f} ms each"},
     }
+
+
+def autograd_step(x, steps: int = 200):
+    """The step as a training loop pays it: torch.func.jvp(sdpa_jvp) and reverse mode through both
+    outputs (one forward launch, one backward launch with both cotangents, plus PyTorch's autograd
+    machinery on the host).  Wall clock per step over `steps` steps."""
+    from semicat_amd import sdpa_jvp
+    leaves = [x[n].detach().requires_grad_(True) for n in NAMES[:6]]
+
+    def step():
+        y, ty = torch.func.jvp(sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+        return torch.autograd.grad([y, ty], leaves, [x["dO"], x["dTO"]])
+
+    for _ in range(20):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
 
 
 def measure_hardware(dev):
@@ -128,6 +187,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache timing over rotating buffer sets")
     ap.add_argument("--no-hardware", action="store_true", help="skip the copy / GEMM measurement of the box")
+    ap.add_argument("--no-autograd", action="store_true",
+                    help="skip timing the step through torch.func.jvp + autograd")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a 256 MiB device copy (reference point for rocprofv3 --pmc byte counters)")
     a = ap.parse_args()
@@ -254,8 +315,11 @@ def main() -> int:
                 dst.copy_(src)
             stream.synchronize()
 
+    # the same step through torch.func.jvp + autograd (host-side machinery included)
+    autograd_ms = None if a.no_autograd else autograd_step(x)
     hardware = None if a.no_hardware else measure_hardware(dev)
     ms_per_step = wall / a.steps * 1e3
+    step_ai = step_flops() / (B * H * (24.0 * L * D * 2 + 16.0 * L))
     tflops = step_flops() / (ms_per_step * 1e-3) / 1e12
 
     # Algorithmic work per (batch, head), e = 2 bytes.  Forward: 6 tile contractions (12 L^2 D flop);
@@ -282,7 +346,7 @@ def main() -> int:
                     "frac": dk["TFLOPs"] / PEAK_BF16_TFLOPS}
     # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
     # this script (scaled by the same counters on the --calib-copy kernel).
-    roofline["traffic"] = MEASURED_TRAFFIC_BYTES.get(dom)
+    roofline["traffic"], roofline["traffic_source"] = measured_traffic(dom)
     roofline["kernel"] = dom
     roofline["ms"] = dk["ms"]
     roofline["algorithmic_bytes"] = dk["bytes"]
@@ -308,6 +372,10 @@ def main() -> int:
                              else "hip-graph replay of one fwd+bwd step",
                    "flop_model": "42*B*H*L^2*D"},
         "pct_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
+        # the step's own roof: min(MFMA peak, flop per algorithmic byte of the step x HBM peak)
+        "pct_of_min_mfma_hbm_roof": 100.0 * tflops / min(PEAK_BF16_TFLOPS, step_ai * PEAK_HBM_GBPS / 1e3),
+        "step_flop_per_byte": step_ai,
+        "autograd_step_ms": autograd_ms,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
         "event_intervals_ms": {"fwd": fwd_raw_ms, "bwd": bwd_raw_ms, "gap_removed_per_kernel": gap_ms},

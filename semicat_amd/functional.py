@@ -15,6 +15,16 @@ How the op is wired (same shape as the reference, functional.py:216-307):
 Beyond the reference: called without forward-mode tangents the reference returns an uninitialised
 ``y`` (functional.py:286-287); here that case is detected and a primal-only kernel computes ``y``
 (and supports reverse mode), so the op is a strict superset.  A missing tangent is treated as zero.
+
+Two wirings of the same op exist; ``AUTOGRAD_WIRING`` selects the one ``sdpa_jvp`` uses:
+
+* ``"fused"`` (default): the dual inputs are unpacked, ONE autograd node (``SDPAFusedFunction``)
+  produces ``y`` and ``t_y`` with one forward launch, and the two are handed back as a dual tensor.
+  Reverse mode then reaches that node once, with the cotangents of both outputs, and runs the
+  backward as ONE launch (the six gradients are accumulated in fp32 and rounded once).
+* ``"reference"``: the reference's three-function arrangement as described above, in which the node
+  of ``y`` and the node of ``t_y`` each launch the backward with their own cotangent and autograd
+  adds the two 16-bit results for q, k, v.
 """
 from __future__ import annotations
 
@@ -25,6 +35,9 @@ import torch.autograd.forward_ad as fwAD
 from torch import Tensor
 
 from . import kernels
+
+
+AUTOGRAD_WIRING = "fused"  # or "reference"
 
 
 def _has_tangent(t: Tensor) -> bool:
@@ -132,6 +145,51 @@ class SDPAFunction(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+class SDPAFusedFunction(torch.autograd.Function):
+    """``(q, k, v, t_q, t_k, t_v) -> (y, t_y)`` as one autograd node: one fused forward launch, and
+    in reverse mode one backward launch that takes the cotangents of both outputs (either may be
+    absent).  Replaces the pair functional.py:52-87 / 216-268 when the caller's dual tensors are
+    unpacked by hand (see ``_sdpa``)."""
+
+    @staticmethod
+    def forward(q, k, v, t_q, t_k, t_v, seq_major=False):
+        y = _empty_output(q, v.shape[-1], seq_major)
+        y, t_y, M, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y, to=torch.empty_like(y),
+                                                         with_li=False)
+        return y, t_y, M, MU
+
+    @staticmethod
+    def setup_context(ctx: Any, inputs: tuple[Any, ...], output: Any) -> Any:
+        y, t_y, M, MU = output
+        ctx.save_for_backward(*inputs[:6], y, t_y, M, MU)
+        ctx.mark_non_differentiable(M, MU)
+        ctx.set_materialize_grads(False)
+
+    @staticmethod
+    def backward(ctx, d_y, d_t_y, *_):
+        if d_y is None and d_t_y is None:
+            return (None,) * 7
+        q, k, v, t_q, t_k, t_v, y, t_y, M, MU = ctx.saved_tensors
+        with torch.no_grad():
+            if d_t_y is None:
+                dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
+                return dq, dk, dv, None, None, None, None
+            grads = SDPAJVPFusedBackwardFunction.apply(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y)
+        return *grads, None
+
+
+class SDPAJVPFusedBackwardFunction(torch.autograd.Function):
+    """Gradients for cotangents on both outputs in one launch (``d_y`` may be None)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y):
+        return kernels.attention_jvp_backward(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, dO=d_y, dTO=d_t_y)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise NotImplementedError("double backward of the attention-JVP op is not implemented")
+
+
 class SDPAPrimalFunction(torch.autograd.Function):
     """The op without forward-mode tangents: plain attention with the primal-only kernels."""
 
@@ -159,8 +217,15 @@ def sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
 @torch._dynamo.disable
 def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool) -> Tensor:
     if _has_tangent(q) or _has_tangent(k) or _has_tangent(v):
-        y, _ = SDPAFunction.apply(q, k, v, seq_major)
-        return y
+        if AUTOGRAD_WIRING == "reference":
+            y, _ = SDPAFunction.apply(q, k, v, seq_major)
+            return y
+        (q, t_q), (k, t_k), (v, t_v) = (fwAD.unpack_dual(t) for t in (q, k, v))
+        t_q = torch.zeros_like(q) if t_q is None else t_q
+        t_k = torch.zeros_like(k) if t_k is None else t_k
+        t_v = torch.zeros_like(v) if t_v is None else t_v
+        y, t_y, _, _ = SDPAFusedFunction.apply(q, k, v, t_q, t_k, t_v, seq_major)
+        return fwAD.make_dual(y, t_y)
     return SDPAPrimalFunction.apply(q, k, v, seq_major)
 
 

@@ -38,6 +38,39 @@ def test_jvp_then_backward_both_cotangents(monkeypatch, dtype, tol):
         assert orc.rel_frobenius(leaf.grad, ref[n]) < tol, n
 
 
+@pytest.mark.parametrize("wiring,launches", [("fused", 1), ("reference", 2)])
+def test_autograd_wirings_agree_and_differ_in_backward_launches(monkeypatch, wiring, launches):
+    """Both wirings of the op give the oracle's gradients; the fused node runs the backward as ONE
+    launch with both cotangents, the reference's arrangement (functional.py:52-87, 216-268) as two
+    launches with one cotangent each."""
+    eager_backend.install(monkeypatch)
+    monkeypatch.setattr(functional, "AUTOGRAD_WIRING", wiring)
+    calls = []
+    real = kernels.attention_jvp_backward
+
+    def spy(*a, dO=None, dTO=None, **kw):
+        calls.append((dO is not None, dTO is not None))
+        return real(*a, dO=dO, dTO=dTO, **kw)
+
+    monkeypatch.setattr(kernels, "attention_jvp_backward", spy)
+    x = orc.make_inputs(2, 2, 24, 40, 16, seed=4)
+    leaves = [_leaf(x[n], torch.float32) for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(functional.sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+    ((y * x["dO"]).sum() + (ty * x["dTO"]).sum()).backward()
+    assert len(calls) == launches
+    assert (True, True) in calls if wiring == "fused" else sorted(calls) == [(False, True), (True, False)]
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    for n, leaf in zip(GRADS, leaves):
+        assert orc.rel_frobenius(leaf.grad, ref[n]) < 2e-5, n
+    # one cotangent only: the other output's branch is skipped (set_materialize_grads(False))
+    calls.clear()
+    leaves = [_leaf(x[n], torch.float32) for n in orc.TENSOR_ORDER[:6]]
+    y, ty = torch.func.jvp(functional.sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+    (y * x["dO"]).sum().backward()
+    assert calls == [(True, False)]
+    assert all(leaf.grad is None for leaf in leaves[3:])
+
+
 @pytest.mark.parametrize("which", ["primal", "tangent"])
 def test_single_cotangent(monkeypatch, which):
     """Only one of the two autograd nodes receives a cotangent (set_materialize_grads(False),

@@ -337,19 +337,25 @@ def test_large_configs_on_head_slices_and_properties(K, B, H, L, D, ps, ts):
 
 
 def test_autograd_end_to_end_on_gpu(K):
-    """torch.func.jvp(sdpa_jvp) then backward through both outputs, all on the HIP kernels."""
-    from semicat_amd import sdpa_jvp, safe_sdpa_jvp
+    """torch.func.jvp(sdpa_jvp) then backward through both outputs, all on the HIP kernels, with both
+    wirings of the op: the fused node (one backward launch, gradients rounded once) and the
+    reference's two nodes (dq, dk, dv are the 16-bit sum of two separately rounded launches)."""
+    from semicat_amd import functional, sdpa_jvp, safe_sdpa_jvp
     B, H, L, D = 2, 4, 128, 64
     x = orc.make_inputs(B, H, L, L, D, seed=8, tangent_scale=0.1, dtype=torch.bfloat16)
     ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
-    leaves = [x[n].cuda().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
-    y, ty = torch.func.jvp(sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
-    loss = (y.float() * x["dO"].cuda().float()).sum() + (ty.float() * x["dTO"].cuda().float()).sum()
-    loss.backward()
-    res = {"O": y.detach().cpu(), "TO": ty.detach().cpu(),
-           **{n: l.grad.cpu() for n, l in zip(GRADS, leaves)}}
-    # dq, dk, dv are the 16-bit sum of two separately rounded launches here
-    assert_parity(res, ref, 1.2e-2, label="autograd")
+    for wiring, tol in (("fused", TOL_16BIT), ("reference", 1.2e-2)):
+        functional.AUTOGRAD_WIRING = wiring
+        try:
+            leaves = [x[n].cuda().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
+            y, ty = torch.func.jvp(sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+            loss = (y.float() * x["dO"].cuda().float()).sum() + (ty.float() * x["dTO"].cuda().float()).sum()
+            loss.backward()
+        finally:
+            functional.AUTOGRAD_WIRING = "fused"
+        res = {"O": y.detach().cpu(), "TO": ty.detach().cpu(),
+               **{n: l.grad.cpu() for n, l in zip(GRADS, leaves)}}
+        assert_parity(res, ref, tol, label=f"autograd, {wiring} wiring")
     # plain call (no tangents) computes attention; [B,S,H,D] fp32 wrapper casts and transposes
     q32 = x["q"].float().cuda().transpose(1, 2).contiguous()
     k32 = x["k"].float().cuda().transpose(1, 2).contiguous()
@@ -366,7 +372,7 @@ def test_autograd_end_to_end_on_gpu(K):
     ((y3.float() * w_o).sum() + (ty3.float() * w_to).sum()).backward()
     res3 = {"O": y3.detach().transpose(1, 2).cpu(), "TO": ty3.detach().transpose(1, 2).cpu(),
             **{n: l.grad.transpose(1, 2).cpu() for n, l in zip(GRADS, bshd)}}
-    assert_parity(res3, ref, 1.2e-2, label="autograd, [B,S,H,D] caller")
+    assert_parity(res3, ref, TOL_16BIT, label="autograd, [B,S,H,D] caller")
 
 
 def test_reference_signature_wrappers(K):
