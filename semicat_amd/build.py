@@ -17,8 +17,8 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libsjvp.so")
 # (source, element types it is compiled for: the unit instantiates its kernels for -DSJVP_T=<type>)
-UNITS = [("sjvp_api.hip", (None,))] + [
-    (name, ("Bf16", "Fp16")) for name in sorted(os.listdir(CSRC)) if name.startswith("sjvp_tu_") and name.endswith(".hip")]
+UNITS = [(name, ("Bf16", "Fp16") if name.startswith("sjvp_tu_") else (None,))
+         for name in sorted(os.listdir(CSRC)) if name.endswith(".hip")]
 SOURCES = [os.path.join(CSRC, name) for name, _ in UNITS]
 HEADERS = sorted(os.path.join(CSRC, n) for n in os.listdir(CSRC) if n.endswith(".hpp")) + [
     os.path.join(os.path.dirname(PKG_DIR), "include", "sjvp.h")]
@@ -74,7 +74,7 @@ def build(verbose: bool = False, jobs: int | None = None) -> str:
     for name, types in UNITS:
         for t in types:
             obj = os.path.join(OBJ_DIR, name[:-4] + (f"_{t}" if t else "") + ".o")
-            define = [f"-DSJVP_T={t}"] if t else [build_id]
+            define = [f"-DSJVP_T={t}"] if t else ([build_id] if name == "sjvp_api.hip" else [])
             cmds.append([hipcc, *HIPCC_FLAGS, *define, "-c", os.path.join(CSRC, name), "-o", obj])
             objs.append(obj)
     jobs = jobs or min(len(cmds), os.cpu_count() or 4, 16)

@@ -34,8 +34,13 @@ inline OutView out_view(void* p, const int64_t* s) {
     return OutView{static_cast<elem_t*>(p), s[0], s[1], s[2]};
 }
 
+inline F32In view32(const void* p, const int64_t* s) {
+    return F32In{static_cast<const float*>(p), s[0], s[1], s[2]};
+}
+inline F32Out out_view32(void* p, const int64_t* s) { return F32Out{static_cast<float*>(p), s[0], s[1], s[2]}; }
+
 int check_common(int B, int H, int Lq, int Lk, int D, int dtype, float scale) {
-    if (dtype != SJVP_BF16 && dtype != SJVP_FP16) return SJVP_ERR_DTYPE;
+    if (dtype != SJVP_BF16 && dtype != SJVP_FP16 && dtype != SJVP_FP32) return SJVP_ERR_DTYPE;
     if (B < 1 || H < 1 || Lq < 1 || Lk < 1) return SJVP_ERR_SHAPE;
     if (D < 16 || D > 128) return SJVP_ERR_HEAD_DIM;
     const int64_t blocks = (int64_t)B * H * ((int64_t)round_up(Lq > Lk ? Lq : Lk, 32) / 32);
@@ -74,6 +79,39 @@ int check_bwd(int parts, const BwdTensors& t, int B, int H, int Lq, int Lk, int 
 int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int Lk, int D,
             const int64_t* strides, float scale, int dtype, void* stream) {
     const bool has_do = t.dO != nullptr, has_g = t.dTO != nullptr;
+    if (dtype == SJVP_FP32) {
+        BwdParamsF32 f{};
+        f.q = view32(t.q, strides + 3 * SJVP_B_Q);
+        f.k = view32(t.k, strides + 3 * SJVP_B_K);
+        f.v = view32(t.v, strides + 3 * SJVP_B_V);
+        f.o = view32(t.o, strides + 3 * SJVP_B_O);
+        if (has_do) f.dO = view32(t.dO, strides + 3 * SJVP_B_DO);
+        f.dq = out_view32(t.dq, strides + 3 * SJVP_B_DQ);
+        f.dk = out_view32(t.dk, strides + 3 * SJVP_B_DK);
+        f.dv = out_view32(t.dv, strides + 3 * SJVP_B_DV);
+        if (has_g) {
+            f.tq = view32(t.tq, strides + 3 * SJVP_B_TQ);
+            f.tk = view32(t.tk, strides + 3 * SJVP_B_TK);
+            f.tv = view32(t.tv, strides + 3 * SJVP_B_TV);
+            f.to = view32(t.to, strides + 3 * SJVP_B_TO);
+            f.dTO = view32(t.dTO, strides + 3 * SJVP_B_DTO);
+            f.dtq = out_view32(t.dtq, strides + 3 * SJVP_B_DTQ);
+            f.dtk = out_view32(t.dtk, strides + 3 * SJVP_B_DTK);
+            f.dtv = out_view32(t.dtv, strides + 3 * SJVP_B_DTV);
+        }
+        f.lse = t.lse;
+        f.mu = t.mu;
+        f.H = H;
+        f.Lq = Lq;
+        f.Lk = Lk;
+        f.D = D;
+        f.Lr = round_up(Lq, 128);
+        f.lse2 = ws;
+        f.s4 = f.lse2 + (size_t)B * H * f.Lr;
+        f.s7d = f.s4 + (size_t)B * H * f.Lr;
+        f.scale = resolve_scale(scale, D);
+        return bwd_f32(f, B * H, has_do, has_g, parts, static_cast<hipStream_t>(stream));
+    }
     const void* ptrs[SJVP_B_COUNT] = {t.q, t.k, t.v, has_g ? t.tq : nullptr, has_g ? t.tk : nullptr,
                                       has_g ? t.tv : nullptr, t.o, has_g ? t.to : nullptr, t.dO, t.dTO,
                                       t.dq, t.dk, t.dv, has_g ? t.dtq : nullptr, has_g ? t.dtk : nullptr,
@@ -157,6 +195,29 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     int rc = check_common(B, H, Lq, Lk, D, dtype, scale);
     if (rc != SJVP_OK) return rc;
 
+    if (dtype == SJVP_FP32) {
+        FwdParamsF32 f{};
+        f.q = view32(q, strides + 3 * SJVP_F_Q);
+        f.k = view32(k, strides + 3 * SJVP_F_K);
+        f.v = view32(v, strides + 3 * SJVP_F_V);
+        if (jvp) {
+            f.tq = view32(tq, strides + 3 * SJVP_F_TQ);
+            f.tk = view32(tk, strides + 3 * SJVP_F_TK);
+            f.tv = view32(tv, strides + 3 * SJVP_F_TV);
+            f.to = out_view32(to, strides + 3 * SJVP_F_TO);
+        }
+        f.o = out_view32(o, strides + 3 * SJVP_F_O);
+        f.lse = lse;
+        f.mu = mu;
+        f.li = li;
+        f.H = H;
+        f.Lq = Lq;
+        f.Lk = Lk;
+        f.D = D;
+        f.Lr = round_up(Lq, 128);
+        f.scale = resolve_scale(scale, D);
+        return fwd_f32(f, B * H, jvp, static_cast<hipStream_t>(stream));
+    }
     const void* ptrs[SJVP_F_COUNT] = {q, k, v, tq, tk, tv, o, to};
     VecCheck vc;
     for (int i = 0; i < SJVP_F_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
@@ -306,7 +367,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_NULL: return "a required pointer is NULL";
         case SJVP_ERR_SHAPE: return "B, H, Lq and Lk must be >= 1 and within the index range";
         case SJVP_ERR_HEAD_DIM: return "head dimension must satisfy 16 <= D <= 128";
-        case SJVP_ERR_DTYPE: return "dtype must be SJVP_BF16 or SJVP_FP16";
+        case SJVP_ERR_DTYPE: return "dtype must be SJVP_BF16, SJVP_FP16 or SJVP_FP32";
         case SJVP_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than sjvp_bwd_workspace_bytes()";
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";

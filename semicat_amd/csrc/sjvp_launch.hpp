@@ -6,6 +6,7 @@
 
 #include "../../include/sjvp.h"
 #include "sjvp_bwd.hpp"
+#include "sjvp_f32.hpp"
 #include "sjvp_fwd.hpp"
 
 namespace sjvp {
@@ -33,5 +34,9 @@ template <typename T> int fwd_any(const FwdParams& p, int grid, bool jvp, hipStr
 template <typename T> int bwd_fused(const BwdParams& p, int BH, bool has_do, bool has_g, hipStream_t stream);
 template <typename T> int bwd_pair_vec(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
 template <typename T> int bwd_pair_any(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
+
+// fp32 correctness mode (vector ALUs): forward, and the row-owned + column-owned backward pair.
+int fwd_f32(const FwdParamsF32& p, int BH, bool jvp, hipStream_t stream);
+int bwd_f32(const BwdParamsF32& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
 
 }  // namespace sjvp

@@ -229,11 +229,13 @@ def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool) -> Tensor:
     return SDPAPrimalFunction.apply(q, k, v, seq_major)
 
 
-def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
+def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Tensor:
     """``[B,S,H,D]`` wrapper that casts to bfloat16 when the inputs are neither bf16 nor fp16 and
-    casts the result back (functional.py:310-332)."""
+    casts the result back (functional.py:310-332).  ``precise=True`` keeps float32 inputs as they are
+    instead: the op then runs in the library's fp32 mode (fp32 tensors and arithmetic throughout,
+    about 1e-6 against fp64, much slower than the MFMA kernels)."""
     orig_dtype = q.dtype
-    if orig_dtype != torch.bfloat16 and orig_dtype != torch.float16:
+    if orig_dtype != torch.bfloat16 and orig_dtype != torch.float16 and not (precise and orig_dtype == torch.float32):
         q = q.to(torch.bfloat16)
         k = k.to(torch.bfloat16)
         v = v.to(torch.bfloat16)

@@ -20,7 +20,9 @@ import torch
 
 from . import _lib
 
-_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16}
+# bf16 / fp16: the MFMA kernels (fp32 accumulation).  float32: the fp32 correctness mode of the library
+# (fp32 tensors and arithmetic throughout, vector ALUs; about 1e-6 against fp64).
+_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16, torch.float32: _lib.SJVP_FP32}
 
 
 def _scale_arg(scale: Optional[float]) -> float:
@@ -82,7 +84,7 @@ def _require_gpu(q: torch.Tensor) -> int:
         raise RuntimeError("semicat_amd kernels run on an AMD GPU only; got a tensor on "
                            f"{q.device} (there is no CPU fallback)")
     if q.dtype not in _DTYPES:
-        raise TypeError(f"attention-JVP kernels support bfloat16 and float16, got {q.dtype}")
+        raise TypeError(f"attention-JVP kernels support bfloat16, float16 and float32, got {q.dtype}")
     return _DTYPES[q.dtype]
 
 

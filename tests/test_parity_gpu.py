@@ -276,6 +276,69 @@ def test_config1_shape_through_the_sixteen_bit_kernels(K):
     assert orc.rel_frobenius(ty.transpose(1, 2).cpu(), ref["TO"]) <= TOL_16BIT
 
 
+TOL_FP32 = 1e-5
+
+
+def test_config1_fp32_mode_meets_1e5(K):
+    """Config 1 (B=2, H=4, L=256, D=64, fp32 N(0,1) inputs, seed 0; unit-normal cotangents on O and TO)
+    on the fp32 mode of the library, through the C ABI: each of the eight outputs within 1e-5
+    (relative Frobenius) of the fp64 math path, which is the bound the reference's fp32 math path
+    meets on the CPU."""
+    x = orc.make_inputs(2, 4, 256, 256, 64, seed=0, dtype=torch.float32)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    assert res["O"].dtype == torch.float32 and res["dtv"].dtype == torch.float32
+    assert_parity(res, ref, TOL_FP32, label="config 1, fp32 mode")
+    check_stats(res, x, 256, 256)
+    # end to end: [B,S,H,D] fp32 tensors through safe_sdpa_jvp(precise=True) under torch.func.jvp
+    from semicat_amd import safe_sdpa_jvp
+    leaves = [x[n].cuda().transpose(1, 2).contiguous().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
+    f = lambda a, b, c: safe_sdpa_jvp(a, b, c, precise=True)
+    y, ty = torch.func.jvp(f, tuple(leaves[:3]), tuple(leaves[3:]))
+    assert y.dtype == torch.float32 and y.is_contiguous()
+    ((y * x["dO"].cuda().transpose(1, 2)).sum() + (ty * x["dTO"].cuda().transpose(1, 2)).sum()).backward()
+    res2 = {"O": y.detach().transpose(1, 2).cpu(), "TO": ty.detach().transpose(1, 2).cpu(),
+            **{n: l.grad.transpose(1, 2).cpu() for n, l in zip(GRADS, leaves)}}
+    assert_parity(res2, ref, TOL_FP32, label="config 1, fp32 mode, autograd")
+
+
+@pytest.mark.parametrize("mode", ["both", "dO", "dTO"])
+@pytest.mark.parametrize("B,H,Lq,Lk,D", [(1, 2, 100, 77, 64), (2, 1, 33, 200, 32), (1, 1, 130, 41, 128),
+                                         (1, 2, 50, 50, 20), (1, 1, 1, 1, 16), (1, 1, 64, 96, 48)])
+def test_fp32_mode_shapes_and_cotangent_modes(K, mode, B, H, Lq, Lk, D):
+    """Ragged lengths, every head-dimension class, odd head dimensions, the three cotangent modes and
+    a [B,S,H,D] caller layout on the fp32 kernels, against the fp64 oracle at 1e-5."""
+    x = orc.make_inputs(B, H, Lq, Lk, D, seed=17, tangent_scale=0.5, dtype=torch.float32)
+    cot = {}
+    if mode != "dTO":
+        cot["dO"] = x["dO"]
+    if mode != "dO":
+        cot["dTO"] = x["dTO"]
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER[:6]], **cot)
+    d = {n: t.cuda().transpose(1, 2).contiguous().transpose(1, 2) for n, t in x.items()}
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    if mode == "dO":
+        g = K.attention_jvp_backward(d["q"], d["k"], d["v"], None, None, None, o, None, lse, None, dO=d["dO"])
+    else:
+        g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                     dO=d["dO"] if mode == "both" else None, dTO=d["dTO"])
+    res = {"O": o.cpu(), "TO": to.cpu(), "lse": lse.cpu(), "mu": mu.cpu(), "li": li.cpu(),
+           **{n: t.cpu() for n, t in zip(GRADS, g) if t is not None}}
+    floor = max(ref[m].norm().item() for m in GRADS)
+    for n in OUTS:
+        if n not in res:
+            continue
+        assert torch.isfinite(res[n]).all(), n
+        err = (res[n].double() - ref[n]).norm().item()
+        scale = ref[n].norm().item()
+        if Lk == 1 and n in GRADS:
+            scale = max(scale, floor)  # a single key: several gradients vanish identically
+        assert err <= TOL_FP32 * max(scale, 1e-30), (n, err / max(scale, 1e-30))
+    check_stats(res, x, Lq, Lk)
+    o2, lse2 = K.attention_forward(d["q"], d["k"], d["v"])
+    assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_FP32
+
+
 def test_bitwise_determinism(K):
     x = orc.make_inputs(2, 2, 200, 136, 64, seed=7, dtype=torch.bfloat16)
     a = run_hip(K, x)
