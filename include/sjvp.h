@@ -19,7 +19,11 @@
  *     L = Lk.  Any [B,S,H,D] caller layout is expressed through the strides.
  *   - dtype: SJVP_BF16 or SJVP_FP16 for every tensor (MFMA kernels; accumulation and softmax are
  *     fp32), or SJVP_FP32: the correctness mode, fp32 tensors and fp32 arithmetic throughout on the
- *     vector ALUs (the reference's fp32 math path, ryu_triton.py:426-454; not tuned for speed).
+ *     vector ALUs (the reference's fp32 math path, ryu_triton.py:426-454; not tuned for speed), or
+ *     SJVP_FP32_BF16: fp32 tensors whose elements are rounded to bf16 as they are loaded, bf16 MFMA
+ *     arithmetic, results stored as fp32, i.e. the casts that functional.py:318-322,330-331 put
+ *     around the op for fp32 callers, folded into it (sjvp_fwd, sjvp_bwd*; not sjvp_rope).  Strides
+ *     are always in elements of the tensors' own storage type.
  *   - Row statistics lse / mu / li are fp32 [B,H,Lr] contiguous with Lr = ceil(Lq/128)*128
  *     (ryu_triton.py:351-358); rows >= Lq receive log(Lk), 0, Lk.
  *   - scale == 0 selects the default 1/sqrt(D) (ryu_triton.py:324-325); a negative or non-finite
@@ -44,14 +48,14 @@ extern "C" {
 
 #define SJVP_VERSION 1
 
-enum sjvp_dtype { SJVP_BF16 = 0, SJVP_FP16 = 1, SJVP_FP32 = 2 };
+enum sjvp_dtype { SJVP_BF16 = 0, SJVP_FP16 = 1, SJVP_FP32 = 2, SJVP_FP32_BF16 = 3 };
 
 enum sjvp_status {
     SJVP_OK = 0,
     SJVP_ERR_NULL = -1,      /* a required pointer is NULL                                   */
     SJVP_ERR_SHAPE = -2,     /* B, H, Lq or Lk < 1, or sizes beyond the 32-bit index range   */
     SJVP_ERR_HEAD_DIM = -3,  /* D < 16 (ryu_triton.py:319-322) or D > 128 (flash_jvp_backward.py:2318) */
-    SJVP_ERR_DTYPE = -4,     /* dtype is none of SJVP_BF16, SJVP_FP16, SJVP_FP32             */
+    SJVP_ERR_DTYPE = -4,     /* dtype is not a member of sjvp_dtype                          */
     SJVP_ERR_WORKSPACE = -5, /* workspace NULL or smaller than sjvp_bwd_workspace_bytes()    */
     SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (status of hipLaunchKernel) */
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */

@@ -9,7 +9,8 @@ from . import build as _build
 
 SJVP_BF16 = 0
 SJVP_FP16 = 1
-SJVP_FP32 = 2  # sjvp_rope only
+SJVP_FP32 = 2
+SJVP_FP32_BF16 = 3  # fp32 tensors, bf16 arithmetic (casts folded into loads and stores)
 
 SJVP_OK = 0
 SJVP_ERR_NULL = -1

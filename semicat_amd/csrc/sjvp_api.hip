@@ -19,19 +19,23 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Whether every row of every tensor starts on a 16-byte boundary (`unit` elements of the tensors'
+// storage type make 16 bytes: 8 for 16-bit storage, 4 for fp32).
 struct VecCheck {
+    int unit = 8;
     bool ok = true;
     void add(const void* p, const int64_t* s) {
         if (!p) return;
-        ok = ok && aligned16(p) && (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0);
+        ok = ok && aligned16(p) && (s[0] % unit == 0) && (s[1] % unit == 0) && (s[2] % unit == 0);
     }
 };
 
-inline TensorView view(const void* p, const int64_t* s) {
-    return TensorView{static_cast<const elem_t*>(p), s[0], s[1], s[2]};
+// Views of the 16-bit kernels.  `m` = 2 for fp32 storage: the kernels address rows in 2-byte units.
+inline TensorView view(const void* p, const int64_t* s, int m = 1) {
+    return TensorView{static_cast<const elem_t*>(p), m * s[0], m * s[1], m * s[2]};
 }
-inline OutView out_view(void* p, const int64_t* s) {
-    return OutView{static_cast<elem_t*>(p), s[0], s[1], s[2]};
+inline OutView out_view(void* p, const int64_t* s, int m = 1) {
+    return OutView{static_cast<elem_t*>(p), m * s[0], m * s[1], m * s[2]};
 }
 
 inline F32In view32(const void* p, const int64_t* s) {
@@ -40,7 +44,7 @@ inline F32In view32(const void* p, const int64_t* s) {
 inline F32Out out_view32(void* p, const int64_t* s) { return F32Out{static_cast<float*>(p), s[0], s[1], s[2]}; }
 
 int check_common(int B, int H, int Lq, int Lk, int D, int dtype, float scale) {
-    if (dtype != SJVP_BF16 && dtype != SJVP_FP16 && dtype != SJVP_FP32) return SJVP_ERR_DTYPE;
+    if (dtype < SJVP_BF16 || dtype > SJVP_FP32_BF16) return SJVP_ERR_DTYPE;
     if (B < 1 || H < 1 || Lq < 1 || Lk < 1) return SJVP_ERR_SHAPE;
     if (D < 16 || D > 128) return SJVP_ERR_HEAD_DIM;
     const int64_t blocks = (int64_t)B * H * ((int64_t)round_up(Lq > Lk ? Lq : Lk, 32) / 32);
@@ -116,27 +120,30 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
                                       has_g ? t.tv : nullptr, t.o, has_g ? t.to : nullptr, t.dO, t.dTO,
                                       t.dq, t.dk, t.dv, has_g ? t.dtq : nullptr, has_g ? t.dtk : nullptr,
                                       has_g ? t.dtv : nullptr};
+    const bool f32io = dtype == SJVP_FP32_BF16;
+    const int m = f32io ? 2 : 1;
     VecCheck vc;
+    vc.unit = f32io ? 4 : 8;
     for (int i = 0; i < SJVP_B_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
 
     BwdParams p{};
-    p.q = view(t.q, strides + 3 * SJVP_B_Q);
-    p.k = view(t.k, strides + 3 * SJVP_B_K);
-    p.v = view(t.v, strides + 3 * SJVP_B_V);
-    p.o = view(t.o, strides + 3 * SJVP_B_O);
-    if (has_do) p.dO = view(t.dO, strides + 3 * SJVP_B_DO);
-    p.dq = out_view(t.dq, strides + 3 * SJVP_B_DQ);
-    p.dk = out_view(t.dk, strides + 3 * SJVP_B_DK);
-    p.dv = out_view(t.dv, strides + 3 * SJVP_B_DV);
+    p.q = view(t.q, strides + 3 * SJVP_B_Q, m);
+    p.k = view(t.k, strides + 3 * SJVP_B_K, m);
+    p.v = view(t.v, strides + 3 * SJVP_B_V, m);
+    p.o = view(t.o, strides + 3 * SJVP_B_O, m);
+    if (has_do) p.dO = view(t.dO, strides + 3 * SJVP_B_DO, m);
+    p.dq = out_view(t.dq, strides + 3 * SJVP_B_DQ, m);
+    p.dk = out_view(t.dk, strides + 3 * SJVP_B_DK, m);
+    p.dv = out_view(t.dv, strides + 3 * SJVP_B_DV, m);
     if (has_g) {
-        p.tq = view(t.tq, strides + 3 * SJVP_B_TQ);
-        p.tk = view(t.tk, strides + 3 * SJVP_B_TK);
-        p.tv = view(t.tv, strides + 3 * SJVP_B_TV);
-        p.to = view(t.to, strides + 3 * SJVP_B_TO);
-        p.dTO = view(t.dTO, strides + 3 * SJVP_B_DTO);
-        p.dtq = out_view(t.dtq, strides + 3 * SJVP_B_DTQ);
-        p.dtk = out_view(t.dtk, strides + 3 * SJVP_B_DTK);
-        p.dtv = out_view(t.dtv, strides + 3 * SJVP_B_DTV);
+        p.tq = view(t.tq, strides + 3 * SJVP_B_TQ, m);
+        p.tk = view(t.tk, strides + 3 * SJVP_B_TK, m);
+        p.tv = view(t.tv, strides + 3 * SJVP_B_TV, m);
+        p.to = view(t.to, strides + 3 * SJVP_B_TO, m);
+        p.dTO = view(t.dTO, strides + 3 * SJVP_B_DTO, m);
+        p.dtq = out_view(t.dtq, strides + 3 * SJVP_B_DTQ, m);
+        p.dtk = out_view(t.dtk, strides + 3 * SJVP_B_DTK, m);
+        p.dtv = out_view(t.dtv, strides + 3 * SJVP_B_DTV, m);
     }
     p.lse = t.lse;
     p.mu = t.mu;
@@ -154,6 +161,7 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (f32io) return bwd_f32io(p, B * H, has_do, has_g, parts, s);
     return dtype == SJVP_BF16 ? bwd_select<Bf16>(p, B * H, has_do, has_g, parts, s)
                               : bwd_select<Fp16>(p, B * H, has_do, has_g, parts, s);
 }
@@ -219,20 +227,23 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
         return fwd_f32(f, B * H, jvp, static_cast<hipStream_t>(stream));
     }
     const void* ptrs[SJVP_F_COUNT] = {q, k, v, tq, tk, tv, o, to};
+    const bool f32io = dtype == SJVP_FP32_BF16;
+    const int m = f32io ? 2 : 1;
     VecCheck vc;
+    vc.unit = f32io ? 4 : 8;
     for (int i = 0; i < SJVP_F_COUNT; ++i) vc.add(ptrs[i], strides + 3 * i);
 
     FwdParams p{};
-    p.q = view(q, strides + 3 * SJVP_F_Q);
-    p.k = view(k, strides + 3 * SJVP_F_K);
-    p.v = view(v, strides + 3 * SJVP_F_V);
+    p.q = view(q, strides + 3 * SJVP_F_Q, m);
+    p.k = view(k, strides + 3 * SJVP_F_K, m);
+    p.v = view(v, strides + 3 * SJVP_F_V, m);
     if (jvp) {
-        p.tq = view(tq, strides + 3 * SJVP_F_TQ);
-        p.tk = view(tk, strides + 3 * SJVP_F_TK);
-        p.tv = view(tv, strides + 3 * SJVP_F_TV);
-        p.to = out_view(to, strides + 3 * SJVP_F_TO);
+        p.tq = view(tq, strides + 3 * SJVP_F_TQ, m);
+        p.tk = view(tk, strides + 3 * SJVP_F_TK, m);
+        p.tv = view(tv, strides + 3 * SJVP_F_TV, m);
+        p.to = out_view(to, strides + 3 * SJVP_F_TO, m);
     }
-    p.o = out_view(o, strides + 3 * SJVP_F_O);
+    p.o = out_view(o, strides + 3 * SJVP_F_O, m);
     p.lse = lse;
     p.mu = mu;
     p.li = li;
@@ -247,6 +258,7 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
 
     const int grid = B * H * p.q_blocks;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (f32io) return fwd_f32io(p, grid, jvp, s);
     // LDS-DMA streaming needs 16-byte aligned rows; anything else takes the register-staged path
     if (p.vec) return dtype == SJVP_BF16 ? fwd_vec<Bf16>(p, grid, jvp, s) : fwd_vec<Fp16>(p, grid, jvp, s);
     return dtype == SJVP_BF16 ? fwd_any<Bf16>(p, grid, jvp, s) : fwd_any<Fp16>(p, grid, jvp, s);
@@ -367,7 +379,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_NULL: return "a required pointer is NULL";
         case SJVP_ERR_SHAPE: return "B, H, Lq and Lk must be >= 1 and within the index range";
         case SJVP_ERR_HEAD_DIM: return "head dimension must satisfy 16 <= D <= 128";
-        case SJVP_ERR_DTYPE: return "dtype must be SJVP_BF16, SJVP_FP16 or SJVP_FP32";
+        case SJVP_ERR_DTYPE: return "dtype must be SJVP_BF16, SJVP_FP16, SJVP_FP32 or SJVP_FP32_BF16";
         case SJVP_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than sjvp_bwd_workspace_bytes()";
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";

@@ -52,7 +52,7 @@ struct RowSmem {
     static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, bool HAS_DO, bool HAS_G>
+template <typename T, int HD, bool HAS_DO, bool HAS_G, bool F32IO = false>
 __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
@@ -82,8 +82,8 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         const elem_t* op = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-            qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
-            oR[c] = load8(op, 16 * c + 8 * hf, p.D, qvalid, vec);
+            qB[c] = load8_io<T, F32IO>(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
+            oR[c] = load8_io<T, F32IO>(op, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
         if constexpr (HAS_G) {
             const elem_t* tqp = p.tq.head(b, h) + (int64_t)qrow * p.tq.sl;
@@ -91,15 +91,15 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
             const elem_t* top = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
-                tqB[c] = load8(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
-                gB[c] = load8(gp, 16 * c + 8 * hf, p.D, qvalid, vec);
-                toR[c] = load8(top, 16 * c + 8 * hf, p.D, qvalid, vec);
+                tqB[c] = load8_io<T, F32IO>(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
+                gB[c] = load8_io<T, F32IO>(gp, 16 * c + 8 * hf, p.D, qvalid, vec);
+                toR[c] = load8_io<T, F32IO>(top, 16 * c + 8 * hf, p.D, qvalid, vec);
             }
         }
         if constexpr (HAS_DO) {
             const elem_t* dop = p.dO.head(b, h) + (int64_t)qrow * p.dO.sl;
 #pragma unroll
-            for (int c = 0; c < KC; ++c) doB[c] = load8(dop, 16 * c + 8 * hf, p.D, qvalid, vec);
+            for (int c = 0; c < KC; ++c) doB[c] = load8_io<T, F32IO>(dop, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
         // Per-lane row statistics; an invalid query lane uses zeros (finite P, results discarded).
         lse2 = qvalid ? p.lse[so] * kLog2e : 0.f;
@@ -143,11 +143,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
 
     auto fill = [&](int st) {
         const int row0 = st * kStageRows;
-        fill_slab<HD>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
-        fill_slab<HD>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, T, F32IO>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, T, F32IO>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
-            fill_slab<HD>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -234,11 +234,11 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     if (!qvalid) return;
     elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;
 #pragma unroll
-    for (int d = 0; d < DT; ++d) store_acc<T>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
+    for (int d = 0; d < DT; ++d) store_acc<T, F32IO>(dqrow, 32 * d, hf, p.D, dq[d], p.scale, vec);
     if constexpr (HAS_G) {
         elem_t* dtqrow = p.dtq.head(b, h) + (int64_t)qrow * p.dtq.sl;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) store_acc<T>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
+        for (int d = 0; d < DT; ++d) store_acc<T, F32IO>(dtqrow, 32 * d, hf, p.D, dtq[d], p.scale, vec);
     }
 }
 
@@ -256,7 +256,7 @@ struct ColSmem {
     static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT>
+template <typename T, int HD, bool HAS_DO, bool HAS_G, bool DO_K, bool DO_V, int DT0, int NDT, bool F32IO = false>
 __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd_col_kernel(
     const BwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -290,16 +290,16 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
         const elem_t* vp = p.v.head(b, h) + (int64_t)krow * p.v.sl;
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-            kB[c] = load8(kp, 16 * c + 8 * hf, p.D, kvalid, vec);
-            if constexpr (DO_K) vB[c] = load8(vp, 16 * c + 8 * hf, p.D, kvalid, vec);
+            kB[c] = load8_io<T, F32IO>(kp, 16 * c + 8 * hf, p.D, kvalid, vec);
+            if constexpr (DO_K) vB[c] = load8_io<T, F32IO>(vp, 16 * c + 8 * hf, p.D, kvalid, vec);
         }
         if constexpr (HAS_G) {
             const elem_t* tkp = p.tk.head(b, h) + (int64_t)krow * p.tk.sl;
             const elem_t* tvp = p.tv.head(b, h) + (int64_t)krow * p.tv.sl;
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
-                tkB[c] = load8(tkp, 16 * c + 8 * hf, p.D, kvalid, vec);
-                if constexpr (DO_K) tvB[c] = load8(tvp, 16 * c + 8 * hf, p.D, kvalid, vec);
+                tkB[c] = load8_io<T, F32IO>(tkp, 16 * c + 8 * hf, p.D, kvalid, vec);
+                if constexpr (DO_K) tvB[c] = load8_io<T, F32IO>(tvp, 16 * c + 8 * hf, p.D, kvalid, vec);
             }
         }
     }
@@ -311,12 +311,12 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
 
     auto fill = [&](int st) {
         const int row0 = st * kStageRows;
-        fill_slab<HD>(ln, stage, qg, p.q.sl, row0, p.Lq, p.D, vec);
+        fill_slab<HD, T, F32IO>(ln, stage, qg, p.q.sl, row0, p.Lq, p.D, vec);
         if constexpr (HAS_G) {
-            fill_slab<HD>(ln, stage + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec);
-            fill_slab<HD>(ln, stage + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + oTQ, tqg, p.tq.sl, row0, p.Lq, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + oG, gg, p.dTO.sl, row0, p.Lq, p.D, vec);
         }
-        if constexpr (HAS_DO) fill_slab<HD>(ln, stage + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec);
+        if constexpr (HAS_DO) fill_slab<HD, T, F32IO>(ln, stage + oDO, dog, p.dO.sl, row0, p.Lq, p.D, vec);
         // Row statistics of the stage (rows < Lr are defined in all four arrays; rows beyond Lq
         // hold finite values and multiply zero rows of Q, Q_dot, G, dO below): the four arrays are
         // dealt to the waves, 32 lanes each.
@@ -444,24 +444,24 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
             elem_t* dkrow = p.dk.head(b, h) + (int64_t)krow * p.dk.sl;
 #pragma unroll
             for (int d = 0; d < NDT; ++d)
-                store_acc<T>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
+                store_acc<T, F32IO>(dkrow, 32 * (DT0 + d), hf, p.D, dk[d], p.scale, vec);
             if constexpr (HAS_G) {
                 elem_t* dtkrow = p.dtk.head(b, h) + (int64_t)krow * p.dtk.sl;
 #pragma unroll
                 for (int d = 0; d < NDT; ++d)
-                    store_acc<T>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
+                    store_acc<T, F32IO>(dtkrow, 32 * (DT0 + d), hf, p.D, dtk[d], p.scale, vec);
             }
         }
         if constexpr (DO_V) {
             elem_t* dvrow = p.dv.head(b, h) + (int64_t)krow * p.dv.sl;
 #pragma unroll
             for (int d = 0; d < NDT; ++d)
-                store_acc<T>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
+                store_acc<T, F32IO>(dvrow, 32 * (DT0 + d), hf, p.D, dv[d], 1.0f, vec);
             if constexpr (HAS_G) {
                 elem_t* dtvrow = p.dtv.head(b, h) + (int64_t)krow * p.dtv.sl;
 #pragma unroll
                 for (int d = 0; d < NDT; ++d)
-                    store_acc<T>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
+                    store_acc<T, F32IO>(dtvrow, 32 * (DT0 + d), hf, p.D, dtv[d], 1.0f, vec);
             }
         }
     }

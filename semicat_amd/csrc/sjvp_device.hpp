@@ -135,6 +135,37 @@ __device__ __forceinline__ u32x4 load8(const elem_t* row, int d, int D, bool val
     return r;
 }
 
+// load8 for either storage: F32IO rows hold fp32 elements (the row pointer is passed as elem_t* with
+// strides counted in 2-byte units, so that row addressing is the same for both storages); they are
+// rounded to T's 16-bit format as they are loaded.  `vec` promises 16-byte alignment and D % 8 == 0.
+template <typename T, bool F32IO>
+__device__ __forceinline__ u32x4 load8_io(const elem_t* row, int d, int D, bool valid, bool vec) {
+    if constexpr (!F32IO) {
+        return load8(row, d, D, valid, vec);
+    } else {
+        const float* fr = reinterpret_cast<const float*>(row);
+        float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (valid) {
+            if (vec) {
+                if (d < D) {
+                    const f32x4 a = *reinterpret_cast<const f32x4*>(fr + d);
+                    const f32x4 b = *reinterpret_cast<const f32x4*>(fr + d + 4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        x[i] = a[i];
+                        x[4 + i] = b[i];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (d + i < D) x[i] = fr[d + i];
+            }
+        }
+        return u32x4{T::pack2(x[0], x[1]), T::pack2(x[2], x[3]), T::pack2(x[4], x[5]), T::pack2(x[6], x[7])};
+    }
+}
+
 // Four consecutive elements (packed in two dwords) to columns d..d+3 of one row, masked at D.
 __device__ __forceinline__ void store4(elem_t* row, int d, int D, u32x2 val, bool vec) {
     if (vec) {
@@ -240,14 +271,15 @@ struct SlabLane {
 // Copy stage rows row0 .. row0+31 of one [L][D] head slice into a slab (swizzled), zero-filled
 // beyond L and beyond D: a synchronous copy through registers that works for any alignment (`vec`
 // selects 16-byte loads when the rows allow them).
-template <int HD>
+template <int HD, typename T = Bf16, bool F32IO = false>
 __device__ __forceinline__ void fill_slab(const SlabLane<HD>& ln, elem_t* slab, const elem_t* g,
                                           int64_t sl, int row0, int L, int D, bool vec) {
 #pragma unroll
     for (int i = 0; i < SlabLane<HD>::N; ++i) {
         if (Slab<HD>::chunks % kThreads != 0 && !ln.on[i]) break;
         const int row = row0 + ln.r[i];
-        *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) = load8(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
+        *reinterpret_cast<u32x4*>(slab + ln.pos8[i]) =
+            load8_io<T, F32IO>(g + (int64_t)row * sl, ln.c8[i], D, row < L, vec);
     }
 }
 
@@ -290,9 +322,26 @@ __device__ __forceinline__ u32x4 pack_b(const f32x16& t, int c) {
 
 // Store one transposed accumulator tile (OUT^T[d][x]: lane = row x of the output tensor, register
 // j = column d0 + 8*(j/4) + 4*hf + j%4) scaled by `mul`, as 16-bit, masked at D.
-template <typename T>
+template <typename T, bool F32IO = false>
 __device__ __forceinline__ void store_acc(elem_t* row, int d0, int hf, int D, const f32x16& acc,
                                           float mul, bool vec) {
+    if constexpr (F32IO) {
+        // fp32 storage: the scaled accumulators leave unrounded
+        float* fr = reinterpret_cast<float*>(row);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int d = d0 + 8 * jj + 4 * hf;
+            const f32x4 val = {acc[4 * jj] * mul, acc[4 * jj + 1] * mul, acc[4 * jj + 2] * mul, acc[4 * jj + 3] * mul};
+            if (vec) {
+                if (d < D) *reinterpret_cast<f32x4*>(fr + d) = val;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (d + i < D) fr[d + i] = val[i];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
         u32x2 val = {T::pack2(acc[4 * jj] * mul, acc[4 * jj + 1] * mul),

@@ -41,7 +41,7 @@ struct FwdSmem {
 // by the exp-sum is unaffected.  This keeps the accumulator rescale out of almost every tile.
 constexpr float kMaxSlack = 6.0f;
 
-template <typename T, int HD, bool JVP>
+template <typename T, int HD, bool JVP, bool F32IO = false>
 __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
@@ -70,11 +70,11 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     {
         const elem_t* qp = p.q.head(b, h) + (int64_t)qrow * p.q.sl;
 #pragma unroll
-        for (int c = 0; c < KC; ++c) qB[c] = load8(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
+        for (int c = 0; c < KC; ++c) qB[c] = load8_io<T, F32IO>(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
         if constexpr (JVP) {
             const elem_t* tqp = p.tq.head(b, h) + (int64_t)qrow * p.tq.sl;
 #pragma unroll
-            for (int c = 0; c < KC; ++c) tqB[c] = load8(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
+            for (int c = 0; c < KC; ++c) tqB[c] = load8_io<T, F32IO>(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
     }
     const elem_t* kg = p.k.head(b, h);
@@ -84,11 +84,11 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
 
     auto fill = [&](int st) {
         const int row0 = st * kStageRows;
-        fill_slab<HD>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
-        fill_slab<HD>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, T, F32IO>(ln, stage, kg, p.k.sl, row0, p.Lk, p.D, vec);
+        fill_slab<HD, T, F32IO>(ln, stage + Slab<HD>::elems, vg, p.v.sl, row0, p.Lk, p.D, vec);
         if constexpr (JVP) {
-            fill_slab<HD>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
-            fill_slab<HD>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + 2 * Slab<HD>::elems, tkg, p.tk.sl, row0, p.Lk, p.D, vec);
+            fill_slab<HD, T, F32IO>(ln, stage + 3 * Slab<HD>::elems, tvg, p.tv.sl, row0, p.Lk, p.D, vec);
         }
     };
 
@@ -247,11 +247,11 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
     if (!qvalid) return;
     elem_t* orow = p.o.head(b, h) + (int64_t)qrow * p.o.sl;
 #pragma unroll
-    for (int d = 0; d < DT; ++d) store_acc<T>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
+    for (int d = 0; d < DT; ++d) store_acc<T, F32IO>(orow, 32 * d, hf, p.D, acc[d], inv_l, vec);
     if constexpr (JVP) {
         elem_t* trow = p.to.head(b, h) + (int64_t)qrow * p.to.sl;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) store_acc<T>(trow, 32 * d, hf, p.D, tacc[d], inv_l, vec);
+        for (int d = 0; d < DT; ++d) store_acc<T, F32IO>(trow, 32 * d, hf, p.D, tacc[d], inv_l, vec);
     }
 }
 

@@ -35,6 +35,11 @@ template <typename T> int bwd_fused(const BwdParams& p, int BH, bool has_do, boo
 template <typename T> int bwd_pair_vec(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
 template <typename T> int bwd_pair_any(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
 
+// fp32 tensors with bf16 arithmetic (the cast folded into the loads and stores): 32-wide kernels.
+// The views carry fp32 pointers cast to elem_t* and strides counted in 2-byte units.
+int fwd_f32io(const FwdParams& p, int grid, bool jvp, hipStream_t stream);
+int bwd_f32io(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);
+
 // fp32 correctness mode (vector ALUs): forward, and the row-owned + column-owned backward pair.
 int fwd_f32(const FwdParamsF32& p, int BH, bool jvp, hipStream_t stream);
 int bwd_f32(const BwdParamsF32& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream);

@@ -62,9 +62,9 @@ class SDPABackwardFunction(torch.autograd.Function):
     """Gradients for the cotangent on the primal output (functional.py:171-213)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, o, do, M):
+    def forward(ctx, q, k, v, o, do, M, arith=None):
         dq, dk, dv, _, _, _ = kernels.attention_jvp_backward(
-            q, k, v, None, None, None, o, None, M, None, dO=do, dTO=None)
+            q, k, v, None, None, None, o, None, M, None, dO=do, dTO=None, arithmetic=arith)
         return dq, dk, dv
 
     @staticmethod
@@ -152,38 +152,41 @@ class SDPAFusedFunction(torch.autograd.Function):
     unpacked by hand (see ``_sdpa``)."""
 
     @staticmethod
-    def forward(q, k, v, t_q, t_k, t_v, seq_major=False):
+    def forward(q, k, v, t_q, t_k, t_v, seq_major=False, arith=None):
         y = _empty_output(q, v.shape[-1], seq_major)
         y, t_y, M, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y, to=torch.empty_like(y),
-                                                         with_li=False)
+                                                         with_li=False, arithmetic=arith)
         return y, t_y, M, MU
 
     @staticmethod
     def setup_context(ctx: Any, inputs: tuple[Any, ...], output: Any) -> Any:
         y, t_y, M, MU = output
         ctx.save_for_backward(*inputs[:6], y, t_y, M, MU)
+        ctx.arith = inputs[7]
         ctx.mark_non_differentiable(M, MU)
         ctx.set_materialize_grads(False)
 
     @staticmethod
     def backward(ctx, d_y, d_t_y, *_):
         if d_y is None and d_t_y is None:
-            return (None,) * 7
+            return (None,) * 8
         q, k, v, t_q, t_k, t_v, y, t_y, M, MU = ctx.saved_tensors
         with torch.no_grad():
             if d_t_y is None:
-                dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
-                return dq, dk, dv, None, None, None, None
-            grads = SDPAJVPFusedBackwardFunction.apply(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y)
-        return *grads, None
+                dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith)
+                return dq, dk, dv, None, None, None, None, None
+            grads = SDPAJVPFusedBackwardFunction.apply(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y,
+                                                       ctx.arith)
+        return *grads, None, None
 
 
 class SDPAJVPFusedBackwardFunction(torch.autograd.Function):
     """Gradients for cotangents on both outputs in one launch (``d_y`` may be None)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y):
-        return kernels.attention_jvp_backward(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, dO=d_y, dTO=d_t_y)
+    def forward(ctx, q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y, arith=None):
+        return kernels.attention_jvp_backward(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, dO=d_y, dTO=d_t_y,
+                                              arithmetic=arith)
 
     @staticmethod
     def backward(ctx, *grads):
@@ -194,16 +197,17 @@ class SDPAPrimalFunction(torch.autograd.Function):
     """The op without forward-mode tangents: plain attention with the primal-only kernels."""
 
     @staticmethod
-    def forward(ctx, q, k, v, seq_major=False):
-        y, M = kernels.attention_forward(q, k, v, o=_empty_output(q, v.shape[-1], seq_major))
+    def forward(ctx, q, k, v, seq_major=False, arith=None):
+        y, M = kernels.attention_forward(q, k, v, o=_empty_output(q, v.shape[-1], seq_major), arithmetic=arith)
         ctx.save_for_backward(q, k, v, y, M)
+        ctx.arith = arith
         return y
 
     @staticmethod
     def backward(ctx, d_y):
         q, k, v, y, M = ctx.saved_tensors
-        dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M)
-        return dq, dk, dv, None
+        dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith)
+        return dq, dk, dv, None, None
 
 
 @torch._dynamo.disable
@@ -215,7 +219,7 @@ def sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
 
 
 @torch._dynamo.disable
-def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool) -> Tensor:
+def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool, arith: Optional[str] = None) -> Tensor:
     if _has_tangent(q) or _has_tangent(k) or _has_tangent(v):
         if AUTOGRAD_WIRING == "reference":
             y, _ = SDPAFunction.apply(q, k, v, seq_major)
@@ -224,24 +228,30 @@ def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool) -> Tensor:
         t_q = torch.zeros_like(q) if t_q is None else t_q
         t_k = torch.zeros_like(k) if t_k is None else t_k
         t_v = torch.zeros_like(v) if t_v is None else t_v
-        y, t_y, _, _ = SDPAFusedFunction.apply(q, k, v, t_q, t_k, t_v, seq_major)
+        y, t_y, _, _ = SDPAFusedFunction.apply(q, k, v, t_q, t_k, t_v, seq_major, arith)
         return fwAD.make_dual(y, t_y)
-    return SDPAPrimalFunction.apply(q, k, v, seq_major)
+    return SDPAPrimalFunction.apply(q, k, v, seq_major, arith)
 
 
 def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Tensor:
-    """``[B,S,H,D]`` wrapper that casts to bfloat16 when the inputs are neither bf16 nor fp16 and
-    casts the result back (functional.py:310-332).  ``precise=True`` keeps float32 inputs as they are
-    instead: the op then runs in the library's fp32 mode (fp32 tensors and arithmetic throughout,
-    about 1e-6 against fp64, much slower than the MFMA kernels)."""
+    """``[B,S,H,D]`` wrapper with the reference's dtype policy (functional.py:310-332): inputs that
+    are neither bf16 nor fp16 are computed in bfloat16 and the result comes back in their dtype.  For
+    float32 inputs the casts are folded into the kernels (elements are rounded to bf16 as they are
+    loaded, results are stored as float32: no cast kernels run around the op); other dtypes are cast
+    with torch.  ``precise=True`` runs float32 inputs in the library's fp32 mode instead (fp32
+    arithmetic throughout, about 1e-6 against fp64, much slower than the MFMA kernels)."""
     orig_dtype = q.dtype
-    if orig_dtype != torch.bfloat16 and orig_dtype != torch.float16 and not (precise and orig_dtype == torch.float32):
+    arith = None
+    if orig_dtype == torch.float32 and not precise and AUTOGRAD_WIRING != "reference" \
+            and k.dtype == torch.float32 and v.dtype == torch.float32:
+        arith = "bf16"
+    elif orig_dtype != torch.bfloat16 and orig_dtype != torch.float16 and not (precise and orig_dtype == torch.float32):
         q = q.to(torch.bfloat16)
         k = k.to(torch.bfloat16)
         v = v.to(torch.bfloat16)
     # The reference returns a [B,S,H,D] view of a [B,H,S,D]-contiguous result, which its callers then
     # copy when they flatten the heads (duo.py:155); here the kernels write [B,S,H,D] memory directly.
-    y = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), seq_major=True).transpose(1, 2)
+    y = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), seq_major=True, arith=arith).transpose(1, 2)
     if y.dtype != orig_dtype:
         y = y.to(orig_dtype)
     return y

@@ -79,12 +79,19 @@ def _check_bhld(name: str, t: torch.Tensor, shape, dtype, device) -> None:
         raise AssertionError(f"{name}: the last dimension must have unit stride")
 
 
-def _require_gpu(q: torch.Tensor) -> int:
+def _require_gpu(q: torch.Tensor, arithmetic: Optional[str] = None) -> int:
+    """The C ABI's dtype tag for the tensors of a call.  ``arithmetic="bf16"`` on float32 tensors
+    selects SJVP_FP32_BF16: elements are rounded to bf16 as the kernels load them and results are
+    stored as float32 (the casts of functional.py:318-322,330-331 folded into the op)."""
     if not q.is_cuda:
         raise RuntimeError("semicat_amd kernels run on an AMD GPU only; got a tensor on "
                            f"{q.device} (there is no CPU fallback)")
     if q.dtype not in _DTYPES:
         raise TypeError(f"attention-JVP kernels support bfloat16, float16 and float32, got {q.dtype}")
+    if arithmetic not in (None, "bf16"):
+        raise ValueError(f"arithmetic must be None or 'bf16', got {arithmetic!r}")
+    if arithmetic == "bf16" and q.dtype == torch.float32:
+        return _lib.SJVP_FP32_BF16
     return _DTYPES[q.dtype]
 
 
@@ -98,12 +105,13 @@ def _stat(buf: Optional[torch.Tensor], name: str, B: int, H: int, Lr: int, devic
 
 
 def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=None, to=None,
-                          lse=None, mu=None, li=None, with_li: bool = True, _plan: bool = False
-                          ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                          lse=None, mu=None, li=None, with_li: bool = True, arithmetic: Optional[str] = None,
+                          _plan: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                      Optional[torch.Tensor]]:
     """Fused forward on [B,H,L,D] views: returns (o, to, lse, mu, li); any of them may be passed in
-    to be filled in place.  ``with_li=False`` skips the LI statistic (returned as None)."""
-    dtype_tag = _require_gpu(q)
+    to be filled in place.  ``with_li=False`` skips the LI statistic (returned as None).
+    ``arithmetic="bf16"`` on float32 tensors: see :func:`_require_gpu`."""
+    dtype_tag = _require_gpu(q, arithmetic)
     B, H, Lq, D = q.shape
     Lk = k.shape[-2]
     if D < 16:
@@ -138,10 +146,10 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=
     return o, to, lse, mu, li
 
 
-def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
-                      ) -> Tuple[torch.Tensor, torch.Tensor]:
+def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None,
+                      arithmetic: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Primal-only forward (tangent contractions compiled out): returns (o, lse)."""
-    dtype_tag = _require_gpu(q)
+    dtype_tag = _require_gpu(q, arithmetic)
     B, H, Lq, D = q.shape
     Lk = k.shape[-2]
     if D < 16:
@@ -169,7 +177,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
                            scale: Optional[float] = None, grads=None, workspace=None,
                            parts: int = _lib.SJVP_BWD_ALL, static_scratch: bool = False,
-                           _plan: bool = False):
+                           arithmetic: Optional[str] = None, _plan: bool = False):
     """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
     Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
     tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
@@ -179,7 +187,7 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
     ``static_scratch=True`` takes the ``sjvp_bwd_noalloc`` entry point instead: the workspace is a
     static device array of the library, so with ``grads`` supplied the call allocates nothing; it
     serves up to ``SJVP_NOALLOC_MAX_ROWS`` statistic rows and calls overlapping on one GPU race."""
-    dtype_tag = _require_gpu(q)
+    dtype_tag = _require_gpu(q, arithmetic)
     if dO is None and dTO is None:
         raise ValueError("attention_jvp_backward needs a cotangent on o, on to, or on both")
     B, H, Lq, D = q.shape

@@ -19,9 +19,16 @@ def _stats(S, TS, Lq, Lk):
     return lse, mu
 
 
+def _reader(arithmetic):
+    """How a launcher sees its inputs: as fp32 values, rounded to bf16 first with arithmetic="bf16"."""
+    if arithmetic == "bf16":
+        return lambda t: None if t is None else t.detach().to(torch.bfloat16).float()
+    return lambda t: None if t is None else t.detach().float()
+
+
 def attention_jvp_forward(q, k, v, tq, tk, tv, scale=None, o=None, to=None, lse=None, mu=None,
-                          li=None, with_li=True):
-    f = lambda t: t.detach().float()
+                          li=None, with_li=True, arithmetic=None):
+    f = _reader(arithmetic)
     qf, kf, vf, tqf, tkf, tvf = map(f, (q, k, v, tq, tk, tv))
     s = scale or 1.0 / math.sqrt(q.shape[-1])
     S = s * qf @ kf.transpose(-1, -2)
@@ -47,10 +54,11 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale=None, o=None, to=None, lse=
     return o, to, lse, mu, None
 
 
-def attention_forward(q, k, v, scale=None, o=None, lse=None):
+def attention_forward(q, k, v, scale=None, o=None, lse=None, arithmetic=None):
+    f = _reader(arithmetic)
     s = scale or 1.0 / math.sqrt(q.shape[-1])
-    S = s * q.detach().float() @ k.detach().float().transpose(-1, -2)
-    O = torch.softmax(S, -1) @ v.detach().float()
+    S = s * f(q) @ f(k).transpose(-1, -2)
+    O = torch.softmax(S, -1) @ f(v)
     lse_, _ = _stats(S, None, q.shape[-2], k.shape[-2])
     o = torch.empty_like(q) if o is None else o
     o.data.copy_(O)
@@ -62,9 +70,9 @@ def attention_forward(q, k, v, scale=None, o=None, lse=None):
 
 
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None, scale=None,
-                           grads=None):
+                           grads=None, arithmetic=None):
     assert dO is not None or dTO is not None
-    f = lambda t: None if t is None else t.detach().float()
+    f = _reader(arithmetic)
     Lq = q.shape[-2]
     s = scale or 1.0 / math.sqrt(q.shape[-1])
     qf, kf, vf, of = f(q), f(k), f(v), f(o)

@@ -108,14 +108,17 @@ def test_plain_forward_and_backward_without_tangents(monkeypatch):
 
 
 def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
-    """[B,S,H,D] in and out, fp32 inputs are computed in bf16 and cast back (functional.py:318-332);
-    inside the op q,k,v are [B,H,S,D] views with strides (S*H*D, D, H*D, 1)."""
+    """[B,S,H,D] in and out; fp32 inputs are computed in bf16 and come back as fp32
+    (functional.py:318-332) with the casts folded into the launch (the launcher gets the fp32 tensors
+    and arithmetic="bf16"); other dtypes are cast with torch.  Inside the op q,k,v are [B,H,S,D] views
+    with strides (S*H*D, D, H*D, 1)."""
     seen = {}
     real = eager_backend.attention_jvp_forward
 
     def spy(q, k, v, *a, **kw):
         seen["strides"] = q.stride()
         seen["dtype"] = q.dtype
+        seen["arithmetic"] = kw.get("arithmetic")
         return real(q, k, v, *a, **kw)
 
     eager_backend.install(monkeypatch)
@@ -123,12 +126,19 @@ def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
     B, S, H, D = 2, 8, 3, 16
     g = torch.Generator().manual_seed(0)
     q, k, v, tq, tk, tv = (torch.randn(B, S, H, D, generator=g) for _ in range(6))
-    y, ty = torch.func.jvp(functional.safe_sdpa_jvp, (q, k, v), (tq, tk, tv))
-    assert y.shape == (B, S, H, D) and y.dtype == torch.float32 and ty.dtype == torch.float32
-    assert seen["strides"] == (S * H * D, D, H * D, 1) and seen["dtype"] == torch.bfloat16
     ref = orc.attention_jvp_autograd(*(t.transpose(1, 2) for t in (q, k, v, tq, tk, tv)))
-    assert orc.rel_frobenius(y.transpose(1, 2), ref["O"]) < 3e-2
-    assert orc.rel_frobenius(ty.transpose(1, 2), ref["TO"]) < 3e-2
+    for dtype, want in ((torch.float32, (torch.float32, "bf16")), (torch.float64, (torch.bfloat16, None))):
+        y, ty = torch.func.jvp(functional.safe_sdpa_jvp, tuple(t.to(dtype) for t in (q, k, v)),
+                               tuple(t.to(dtype) for t in (tq, tk, tv)))
+        assert y.shape == (B, S, H, D) and y.dtype == dtype and ty.dtype == dtype
+        assert seen["strides"] == (S * H * D, D, H * D, 1)
+        assert (seen["dtype"], seen["arithmetic"]) == want
+        assert orc.rel_frobenius(y.transpose(1, 2), ref["O"]) < 3e-2
+        assert orc.rel_frobenius(ty.transpose(1, 2), ref["TO"]) < 3e-2
+    # precise=True keeps fp32 tensors and fp32 arithmetic
+    y, ty = torch.func.jvp(lambda a, b, c: functional.safe_sdpa_jvp(a, b, c, precise=True), (q, k, v), (tq, tk, tv))
+    assert (seen["dtype"], seen["arithmetic"]) == (torch.float32, None)
+    assert orc.rel_frobenius(ty.transpose(1, 2), ref["TO"]) < 2e-5
 
 
 def test_through_a_module_with_scalar_time_tangent(monkeypatch):

@@ -339,6 +339,68 @@ def test_fp32_mode_shapes_and_cotangent_modes(K, mode, B, H, Lq, Lk, D):
     assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_FP32
 
 
+@pytest.mark.parametrize("mode", ["both", "dO", "dTO"])
+@pytest.mark.parametrize("B,H,Lq,Lk,D,seq_major", [(2, 3, 128, 128, 64, True), (1, 2, 200, 150, 64, False),
+                                                   (1, 2, 70, 130, 128, True), (1, 1, 50, 50, 20, False),
+                                                   (2, 1, 33, 41, 32, True)])
+def test_fp32_tensors_with_bf16_arithmetic(K, mode, B, H, Lq, Lk, D, seq_major):
+    """The casts that the reference puts around the op for fp32 callers (functional.py:318-322, 330-331)
+    folded into the kernels: fp32 tensors handed over as they are with arithmetic="bf16" give, up to
+    the final rounding of the outputs (stored as fp32 here, as bf16 there), what the bf16 kernels give
+    on the pre-cast tensors, and both meet the bf16 gate against the fp64 oracle on the rounded inputs."""
+    x32 = orc.make_inputs(B, H, Lq, Lk, D, seed=23, tangent_scale=0.3, dtype=torch.float32)
+    xr = {n: t.to(torch.bfloat16) for n, t in x32.items()}
+    cot = {}
+    if mode != "dTO":
+        cot["dO"] = xr["dO"]
+    if mode != "dO":
+        cot["dTO"] = xr["dTO"]
+    ref = orc.attention_jvp_autograd(*[xr[n] for n in orc.TENSOR_ORDER[:6]], **cot)
+    lay = (lambda t: t.cuda().transpose(1, 2).contiguous().transpose(1, 2)) if seq_major else (lambda t: t.cuda())
+    d = {n: lay(t) for n, t in x32.items()}
+    o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], arithmetic="bf16")
+    assert o.dtype == torch.float32 and lse.dtype == torch.float32
+    if mode == "dO":
+        g = K.attention_jvp_backward(d["q"], d["k"], d["v"], None, None, None, o, None, lse, None, dO=d["dO"],
+                                     arithmetic="bf16")
+    else:
+        g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                     dO=d["dO"] if mode == "both" else None, dTO=d["dTO"], arithmetic="bf16")
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g) if t is not None}}
+    for n, t in res.items():
+        assert t.dtype == torch.float32 and torch.isfinite(t).all(), n
+        if seq_major and n in GRADS:  # gradients take the strides of their inputs
+            assert t.stride() == d["q" if n in ("dq", "dtq") else "k"].stride()
+    assert_parity(res, ref, TOL_16BIT, names=[n for n in OUTS if n in res],
+                  label=f"fp32 tensors, bf16 arithmetic {(B, H, Lq, Lk, D)} {mode}")
+    o2, lse2 = K.attention_forward(d["q"], d["k"], d["v"], arithmetic="bf16")
+    assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_16BIT
+
+
+def test_safe_sdpa_jvp_runs_no_cast_kernels_for_fp32_callers(K):
+    """safe_sdpa_jvp on fp32 [B,S,H,D] tensors under torch.func.jvp and reverse mode: same results as
+    casting to bf16 first, and the only kernels launched are the library's (forward, backward)."""
+    from semicat_amd import safe_sdpa_jvp
+    B, H, L, D = 2, 4, 128, 64
+    x32 = orc.make_inputs(B, H, L, L, D, seed=29, tangent_scale=0.1, dtype=torch.float32)
+    ref = orc.attention_jvp_autograd(*[x32[n].to(torch.bfloat16) for n in orc.TENSOR_ORDER])
+    leaves = [x32[n].cuda().transpose(1, 2).contiguous().requires_grad_(True) for n in orc.TENSOR_ORDER[:6]]
+    w_o, w_to = x32["dO"].cuda().transpose(1, 2).contiguous(), x32["dTO"].cuda().transpose(1, 2).contiguous()
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y, ty = torch.func.jvp(safe_sdpa_jvp, tuple(leaves[:3]), tuple(leaves[3:]))
+        grads = torch.autograd.grad([y, ty], leaves, [w_o, w_to])
+        torch.cuda.synchronize()
+    names = [e.key for e in prof.key_averages() if e.device_type == torch.autograd.DeviceType.CUDA]
+    print("[kernels launched]", names, flush=True)
+    foreign = [n for n in names if "sjvp" not in n and "Memcpy" not in n and "Memset" not in n]
+    assert not foreign, foreign
+    assert y.dtype == torch.float32 and y.is_contiguous()
+    res = {"O": y.detach().transpose(1, 2).cpu(), "TO": ty.detach().transpose(1, 2).cpu(),
+           **{n: g_.transpose(1, 2).cpu() for n, g_ in zip(GRADS, grads)}}
+    assert_parity(res, ref, TOL_16BIT, label="safe_sdpa_jvp, fp32 caller")
+
+
 def test_bitwise_determinism(K):
     x = orc.make_inputs(2, 2, 200, 136, 64, seed=7, dtype=torch.bfloat16)
     a = run_hip(K, x)
