@@ -60,7 +60,8 @@ enum sjvp_status {
     SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (status of hipLaunchKernel) */
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
     SJVP_ERR_PARTS = -8,     /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
-    SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16 */
+    SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16;
+                                sjvp_fwd_rotary / sjvp_bwd_rotary: a shape, dtype or table they do not serve */
     SJVP_ERR_SCALE = -10,    /* scale negative, infinite or NaN (0 selects the default)      */
     SJVP_ERR_SCRATCH = -11   /* sjvp_bwd_noalloc: problem beyond SJVP_NOALLOC_MAX_ROWS, or no static scratch on this device */
 };
@@ -115,6 +116,31 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
                    void* dtq, void* dtk, void* dtv, void* workspace, size_t workspace_bytes, int B,
                    int H, int Lq, int Lk, int D, const int64_t* strides /* [SJVP_B_COUNT*3] */,
                    float scale, int dtype, void* stream);
+
+/*
+ * sjvp_fwd() / sjvp_bwd() with the rotary position embedding of semicat/net/duo.py:45-55 folded in:
+ * q, k (and tq, tk) are given UNROTATED; the kernels rotate them as they load them (position = row
+ * index, column j < 32 paired with j + 32, the rotation of sjvp_rope() with rot_dim = D = 64), and the
+ * backward returns the gradients with respect to the unrotated tensors (dq, dk, dtq, dtk pass through
+ * the inverse rotation on their way out).  This removes the separate rotary launches and the rotated
+ * copies of q, k in front of the op.  Served shapes: D = 64, Lk <= 128 (one workgroup walks a head's
+ * keys once), SJVP_BF16 / SJVP_FP16 tensors with 16-byte aligned rows; cos, sin: fp32
+ * [table_rows][32] with row stride cs_stride (multiple of 4), 16-byte aligned, table_rows >=
+ * max(Lq, Lk).  Anything else returns SJVP_ERR_ROTARY before a launch (use sjvp_rope() + sjvp_fwd()).
+ * sjvp_bwd_rotary() needs no workspace.  No counterpart in the reference, which rotates with separate
+ * fp32 PyTorch operations.
+ */
+int sjvp_fwd_rotary(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                    const void* tv, void* o, void* to, float* lse, float* mu, float* li, int B, int H,
+                    int Lq, int Lk, int D, const int64_t* strides /* [SJVP_F_COUNT*3] */, float scale,
+                    int dtype, const float* cos, const float* sin, int64_t cs_stride, int table_rows,
+                    void* stream);
+int sjvp_bwd_rotary(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                    const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+                    const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq, void* dtk,
+                    void* dtv, int B, int H, int Lq, int Lk, int D,
+                    const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, const float* cos,
+                    const float* sin, int64_t cs_stride, int table_rows, void* stream);
 
 /*
  * sjvp_bwd() with the workspace taken from a static device array inside the library instead of a

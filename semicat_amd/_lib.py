@@ -34,7 +34,7 @@ F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
 B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
-EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_noalloc", "sjvp_bwd_workspace_bytes", "sjvp_rope",
+EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_noalloc", "sjvp_fwd_rotary", "sjvp_bwd_rotary", "sjvp_bwd_workspace_bytes", "sjvp_rope",
            "sjvp_strerror", "sjvp_version", "sjvp_build_id")
 
 _lock = threading.Lock()
@@ -69,6 +69,12 @@ def load() -> ctypes.CDLL:
             lib.sjvp_bwd_noalloc.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [i] * 5 +
                                              [i64p, ctypes.c_float, i, vp])
             lib.sjvp_bwd_noalloc.restype = i
+            rot = [vp, vp, ctypes.c_int64, i]  # cos, sin, row stride, rows
+            lib.sjvp_fwd_rotary.argtypes = ([vp] * 8 + [vp] * 3 + [i] * 5 + [i64p, ctypes.c_float, i] + rot + [vp])
+            lib.sjvp_fwd_rotary.restype = i
+            lib.sjvp_bwd_rotary.argtypes = ([vp] * 10 + [vp] * 2 + [vp] * 6 + [i] * 5 + [i64p, ctypes.c_float, i] +
+                                            rot + [vp])
+            lib.sjvp_bwd_rotary.restype = i
             lib.sjvp_bwd_parts.argtypes = [i] + lib.sjvp_bwd.argtypes
             lib.sjvp_bwd_parts.restype = i
             lib.sjvp_bwd_workspace_bytes.argtypes = [i] * 6

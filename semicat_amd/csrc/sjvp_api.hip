@@ -53,6 +53,17 @@ int check_common(int B, int H, int Lq, int Lk, int D, int dtype, float scale) {
     return SJVP_OK;
 }
 
+// The folded rotary embedding serves the shapes of the single-workgroup kernels: head dimension 64
+// rotated as a whole, a key axis of at most 128, 16-bit tensors with 16-byte aligned rows.
+int check_rotary(const float* cos, const float* sin, int64_t cs_stride, int table_rows, int Lq, int Lk, int D,
+                 int dtype) {
+    if (!cos || !sin) return SJVP_ERR_NULL;
+    if (dtype != SJVP_BF16 && dtype != SJVP_FP16) return SJVP_ERR_ROTARY;
+    if (D != 64 || Lk > kOwned16 || table_rows < (Lq > Lk ? Lq : Lk)) return SJVP_ERR_ROTARY;
+    if (!aligned16(cos) || !aligned16(sin) || cs_stride % 4 != 0 || cs_stride < 32) return SJVP_ERR_ROTARY;
+    return SJVP_OK;
+}
+
 inline float resolve_scale(float scale, int D) { return scale > 0.f ? scale : 1.0f / sqrtf((float)D); }
 
 // Kernel selection of the backward: the single launch where it fits, else the row + column pair.
@@ -81,7 +92,8 @@ int check_bwd(int parts, const BwdTensors& t, int B, int H, int Lq, int Lk, int 
 
 // Launches of the backward on a validated problem; `ws` holds 3 * B * H * Lr floats.
 int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int Lk, int D,
-            const int64_t* strides, float scale, int dtype, void* stream) {
+            const int64_t* strides, float scale, int dtype, void* stream,
+            RopeTables rope = RopeTables{nullptr, nullptr, 0, 0}) {
     const bool has_do = t.dO != nullptr, has_g = t.dTO != nullptr;
     if (dtype == SJVP_FP32) {
         BwdParamsF32 f{};
@@ -159,6 +171,8 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
     p.s7d = p.s4 + (size_t)B * H * p.Lr;
     p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
+    p.rope = rope;
+    if (rope.cos && (!p.vec || parts != SJVP_BWD_ALL)) return SJVP_ERR_ROTARY;  // the single launch only
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (f32io) return bwd_f32io(p, B * H, has_do, has_g, parts, s);
@@ -176,6 +190,10 @@ static __device__ __align__(256) __attribute__((used)) float scratch[3 * (size_t
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 float* g_scratch_ptr[kMaxDevices] = {};
+
+int fwd_impl(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
+             void* o, void* to, float* lse, float* mu, float* li, int B, int H, int Lq, int Lk, int D,
+             const int64_t* strides, float scale, int dtype, RopeTables rope, void* stream);
 
 int static_scratch(float** out) {
     int dev = -1;
@@ -197,6 +215,27 @@ extern "C" {
 int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,
              const void* tv, void* o, void* to, float* lse, float* mu, float* li, int B, int H,
              int Lq, int Lk, int D, const int64_t* strides, float scale, int dtype, void* stream) {
+    return fwd_impl(q, k, v, tq, tk, tv, o, to, lse, mu, li, B, H, Lq, Lk, D, strides, scale, dtype,
+                    RopeTables{nullptr, nullptr, 0, 0}, stream);
+}
+
+int sjvp_fwd_rotary(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                    const void* tv, void* o, void* to, float* lse, float* mu, float* li, int B, int H,
+                    int Lq, int Lk, int D, const int64_t* strides, float scale, int dtype,
+                    const float* cos, const float* sin, int64_t cs_stride, int table_rows, void* stream) {
+    const int rc = check_rotary(cos, sin, cs_stride, table_rows, Lq, Lk, D, dtype);
+    if (rc != SJVP_OK) return rc;
+    return fwd_impl(q, k, v, tq, tk, tv, o, to, lse, mu, li, B, H, Lq, Lk, D, strides, scale, dtype,
+                    RopeTables{cos, sin, cs_stride, table_rows}, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+int fwd_impl(const void* q, const void* k, const void* v, const void* tq, const void* tk, const void* tv,
+             void* o, void* to, float* lse, float* mu, float* li, int B, int H, int Lq, int Lk, int D,
+             const int64_t* strides, float scale, int dtype, RopeTables rope, void* stream) {
     if (!q || !k || !v || !o || !lse || !strides) return SJVP_ERR_NULL;
     const bool jvp = tq || tk || tv || to || mu;
     if (jvp && (!tq || !tk || !tv || !to || !mu)) return SJVP_ERR_NULL;
@@ -255,6 +294,8 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     p.q_blocks = p.Lr / kOwned;  // covers every statistic row below Lr
     p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
+    p.rope = rope;
+    if (rope.cos && !p.vec) return SJVP_ERR_ROTARY;
 
     const int grid = B * H * p.q_blocks;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -263,6 +304,10 @@ int sjvp_fwd(const void* q, const void* k, const void* v, const void* tq, const 
     if (p.vec) return dtype == SJVP_BF16 ? fwd_vec<Bf16>(p, grid, jvp, s) : fwd_vec<Fp16>(p, grid, jvp, s);
     return dtype == SJVP_BF16 ? fwd_any<Bf16>(p, grid, jvp, s) : fwd_any<Fp16>(p, grid, jvp, s);
 }
+
+}  // namespace
+
+extern "C" {
 
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype) {
     (void)Lk;
@@ -294,6 +339,22 @@ int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const
         (reinterpret_cast<uintptr_t>(workspace) & 3u))
         return SJVP_ERR_WORKSPACE;
     return run_bwd(parts, t, static_cast<float*>(workspace), B, H, Lq, Lk, D, strides, scale, dtype, stream);
+}
+
+int sjvp_bwd_rotary(const void* q, const void* k, const void* v, const void* tq, const void* tk,
+                    const void* tv, const void* o, const void* to, const void* dO, const void* dTO,
+                    const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq, void* dtk,
+                    void* dtv, int B, int H, int Lq, int Lk, int D, const int64_t* strides, float scale,
+                    int dtype, const float* cos, const float* sin, int64_t cs_stride, int table_rows,
+                    void* stream) {
+    const BwdTensors t{q, k, v, tq, tk, tv, o, to, dO, dTO, lse, mu, dq, dk, dv, dtq, dtk, dtv};
+    int rc = check_bwd(SJVP_BWD_ALL, t, B, H, Lq, Lk, D, strides, scale, dtype);
+    if (rc != SJVP_OK) return rc;
+    rc = check_rotary(cos, sin, cs_stride, table_rows, Lq, Lk, D, dtype);
+    if (rc != SJVP_OK) return rc;
+    // the single-launch backward, which these shapes take, uses no workspace
+    return run_bwd(SJVP_BWD_ALL, t, nullptr, B, H, Lq, Lk, D, strides, scale, dtype, stream,
+                   RopeTables{cos, sin, cs_stride, table_rows});
 }
 
 int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq, const void* tk,
@@ -386,7 +447,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
         case SJVP_ERR_SCALE: return "scale must be finite and >= 0 (0 selects 1/sqrt(D))";
         case SJVP_ERR_SCRATCH: return "sjvp_bwd_noalloc: B * H * ceil(Lq/128)*128 exceeds SJVP_NOALLOC_MAX_ROWS, or the static scratch could not be located on this device";
-        case SJVP_ERR_ROTARY: return "sjvp_rope: n must be 1..4, rot_dim even and 2 <= rot_dim <= D, and bf16 / fp16 must not be mixed";
+        case SJVP_ERR_ROTARY: return "rotary embedding: sjvp_rope needs n in 1..4, rot_dim even with 2 <= rot_dim <= D, and no mix of bf16 and fp16; sjvp_fwd_rotary / sjvp_bwd_rotary need D = 64, Lk <= 128, bf16 or fp16 tensors with 16-byte aligned rows, and 16-byte aligned fp32 tables of at least max(Lq, Lk) rows with a row stride that is a multiple of 4";
         default: return "unknown sjvp status";
     }
 }

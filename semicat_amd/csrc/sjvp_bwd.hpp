@@ -39,6 +39,7 @@ struct BwdParams {
     int q_blocks, k_blocks;  // workgroups per (batch, head) along the owned axis
     float scale;
     int vec;
+    RopeTables rope;  // q, k (and tangents) are rotated as they are loaded, their gradients rotated back
 };
 
 // ---------------------------------------------------------------------------------------------

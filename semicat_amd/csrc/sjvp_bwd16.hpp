@@ -44,9 +44,13 @@ struct Fused16Smem {
     static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G>
+// ROPE: q, k and their tangents are rotated by p.rope once they are in LDS (own K, K_dot rows in the
+// prologue, each stage's Q, Q_dot slabs by the threads that do not form row sums), and the gradients
+// dQ, dQ_dot, dK, dK_dot go back through the inverse rotation on their way out (head dimension 64).
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool ROPE = false>
 __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdParams p) {
     static_assert(HD <= 64, "the accumulators of four gradients must fit the register file");
+    static_assert(!ROPE || HD == 64, "the folded rotation covers a head dimension of 64");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     using SM = Fused16Smem<HD, R, HAS_DO, HAS_G>;
     constexpr int SE = Slab<HD>::elems;
@@ -354,7 +358,10 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if (half == 1 && !HAS_G) return;
         const int r = t / CH, c = t % CH;
         if (r < kStageRows && row0 + r < p.Lq && 8 * c < p.D) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(qstage + half * kStageRows * SM::qpitch + r * SM::qpitch + 8 * c);
+            const elem_t* srow = qstage + half * kStageRows * SM::qpitch + r * SM::qpitch;
+            u32x4 v = *reinterpret_cast<const u32x4*>(srow + 8 * c);
+            if constexpr (ROPE)
+                v = rope8_inverse_chunk<T>(v, *reinterpret_cast<const u32x4*>(srow + 8 * (c ^ 4)), p.rope, row0 + r, c);
             elem_t* dst = (half == 0 ? p.dq.head(b, h) + (int64_t)(row0 + r) * p.dq.sl
                                      : p.dtq.head(b, h) + (int64_t)(row0 + r) * p.dtq.sl) + 8 * c;
             __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
@@ -366,6 +373,24 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     wait_stages<SPT>(0);
     __syncthreads();
     if (issued < ns) issue_next();
+    // ROPE: Q (, Q_dot) of a landed stage, one item per thread of the upper half of the workgroup
+    auto rotate_stage = [&](elem_t* slot, int row0) {
+        if constexpr (ROPE) {
+            const int it = tid - 256;
+            if (it >= 0 && it < 128) rope_slab_item<T>(slot, it, p.rope, row0, 1.0f);
+            else if (HAS_G && it >= 128) rope_slab_item<T>(slot + oTQ, it - 128, p.rope, row0, 1.0f);
+        }
+    };
+    if constexpr (ROPE) {
+        // own K (, K_dot): slabs of 32 keys, 128 items each
+        constexpr int items = (HAS_G ? 8 : 4) * 128;
+#pragma unroll
+        for (int it = tid; it < items; it += kThreads16) {
+            const int slab = it >> 7;
+            rope_slab_item<T>(ownK + slab * SE, it & 127, p.rope, 32 * (slab & 3), 1.0f);
+        }
+        __syncthreads();
+    }
     {
         const int r = 16 * (wave & 1) + n;
         const int sidx = wave >> 1;
@@ -377,6 +402,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
     }
     row_sums(ring);
+    rotate_stage(ring, 0);
     for (int i = 0; i < ns; ++i) {
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
@@ -387,7 +413,10 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if (wave_active) tile(slot);
         if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
         __syncthreads();
-        if (i + 1 < ns) row_sums(ring + ((i + 1) % R) * SM::slot);
+        if (i + 1 < ns) {
+            row_sums(ring + ((i + 1) % R) * SM::slot);
+            rotate_stage(ring + ((i + 1) % R) * SM::slot, (i + 1) * kStageRows);
+        }
         if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
         else row_outputs(i * kStageRows, std::false_type{});
     }
@@ -396,9 +425,10 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = wave * 16;
-    store_tile16<T, HD>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane);
+    store_tile16<T, HD, ROPE>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane, &p.rope);
     if constexpr (HAS_G)
-        store_tile16<T, HD>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane);
+        store_tile16<T, HD, ROPE>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane,
+                                  &p.rope);
     store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
     if constexpr (HAS_G)
         store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);

@@ -111,6 +111,14 @@ struct OutView {
     __device__ __forceinline__ elem_t* head(int b, int h) const { return ptr + b * sb + h * sh; }
 };
 
+// cos / sin tables of a rotary position embedding folded into a kernel (see sjvp_w16.hpp)
+struct RopeTables {
+    const float* cos;  // [rows][32] fp32, row stride cs (multiple of 4, 16-byte aligned base); null: no rotation
+    const float* sin;
+    int64_t cs;
+    int rows;          // rows of the tables (positions beyond are clamped; their data is zero padding)
+};
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -25,6 +25,7 @@ struct FwdParams {
     int q_blocks;  // workgroups per (batch, head): Lr / (32 * waves per workgroup)
     float scale;
     int vec;  // all tensors 16-byte aligned, strides % 8 == 0, D % 8 == 0
+    RopeTables rope;  // rotation of q, k (and their tangents) as they are loaded; cos == null: none
 };
 
 // LDS layout: one stage of K, V (, K_dot, V_dot) slabs.

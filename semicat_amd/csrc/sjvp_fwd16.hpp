@@ -31,8 +31,13 @@ struct Fwd16Smem {
     static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool JVP, int OCC, int SPB = 1>
+// ROPE: q, k and their tangents are rotated by p.rope as they are loaded (head dimension 64, one
+// stage per barrier): the own rows in registers, each stage's K (, K_dot) slab in place in LDS.  Meant
+// for key axes that one workgroup per (batch, head) walks once (every workgroup rotates the K rows it
+// streams).
+template <typename T, int HD, int R, bool JVP, int OCC, int SPB = 1, bool ROPE = false>
 __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams p) {
+    static_assert(!ROPE || (HD == 64 && SPB == 1), "the folded rotation covers HD = 64, one stage per barrier");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     using SM = Fwd16Smem<HD, R, JVP, SPB>;
     elem_t* own = reinterpret_cast<elem_t*>(smem_raw) + SM::own_off;
@@ -105,7 +110,21 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         const int r = 16 * (wave & 1) + n;
         read_b_operands16<HD>(qB, own + (wave >> 1) * SE, r, g);
         if constexpr (JVP) read_b_operands16<HD>(tqB, own + (4 + (wave >> 1)) * SE, r, g);
+        if constexpr (ROPE) {
+            // the lane's two operands are columns 8g.. and 32 + 8g.. of its query: a rotation pair
+            rope8<T>(qB[0], qB[1], p.rope, qrow, g, 1.0f);
+            if constexpr (JVP) rope8<T>(tqB[0], tqB[1], p.rope, qrow, g, 1.0f);
+        }
     }
+    // ROPE: rotate the K (, K_dot) slab of a landed stage in place; 128 items per slab
+    auto rotate_stage = [&](elem_t* slot, int k0) {
+        if constexpr (ROPE) {
+            if (tid < 128) rope_slab_item<T>(slot, tid, p.rope, k0, 1.0f);
+            else if (JVP && tid < 256) rope_slab_item<T>(slot + 2 * SE, tid - 128, p.rope, k0, 1.0f);
+            __syncthreads();
+        }
+    };
+    rotate_stage(ring, 0);
     if constexpr (SPB == 2) {
         // the operands must have arrived in registers before the copies below overwrite their slots
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -194,6 +213,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
 #pragma unroll
             for (int u = 0; u < SPB; ++u)
                 if (issued < ns) issue_next();
+            rotate_stage(ring + (i % R) * SM::slot, i * kStageRows);
         }
         if (!wave_active) continue;
 #pragma unroll

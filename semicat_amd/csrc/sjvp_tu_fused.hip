@@ -9,6 +9,11 @@ constexpr int kRingFused = 3;
 
 template <typename T, int HD, bool HAS_DO, bool HAS_G>
 int fused_mode(const BwdParams& p, int BH, hipStream_t stream) {
+    if constexpr (HD == 64) {
+        if (p.rope.cos)  // rotary embedding folded in
+            return launch(bwd_fused16_kernel<T, HD, kRingFused, HAS_DO, HAS_G, true>, BH,
+                          Fused16Smem<HD, kRingFused, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
+    }
     return launch(bwd_fused16_kernel<T, HD, kRingFused, HAS_DO, HAS_G>, BH,
                   Fused16Smem<HD, kRingFused, HAS_DO, HAS_G>::bytes, stream, p, kThreads16);
 }

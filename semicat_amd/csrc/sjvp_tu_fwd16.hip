@@ -17,6 +17,15 @@ int fwd16_hd(const FwdParams& p, int grid, bool jvp, hipStream_t stream) {
     // two stages in flight and at most 128 registers: two workgroups (sixteen waves) share a CU, which
     // overlaps one's copies with the other's arithmetic; HD = 128 needs the whole register budget
     constexpr int OCC = HD == 128 ? 2 : 4;
+    if constexpr (HD == 64) {
+        if (p.rope.cos) {  // rotary embedding folded in (short key axes only, checked by the caller)
+            if (jvp)
+                return launch(fwd16_kernel<T, HD, kRingJvp, true, OCC, 1, true>, grid,
+                              Fwd16Smem<HD, kRingJvp, true>::bytes, stream, p, kThreads16);
+            return launch(fwd16_kernel<T, HD, kRingPrimal, false, OCC, 1, true>, grid,
+                          Fwd16Smem<HD, kRingPrimal, false>::bytes, stream, p, kThreads16);
+        }
+    }
     if (p.Lk >= kFwdPairedFrom) {
         // long key axes: two stages per barrier over a ring of four slots in the same LDS footprint
         if (jvp)

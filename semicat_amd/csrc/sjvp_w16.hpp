@@ -186,6 +186,53 @@ __device__ __forceinline__ float sum8(float v) {
     return v;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Rotary position embedding folded into the attention kernels (head dimension 64, rotation over the
+// whole head: column j < 32 of a row is paired with column j + 32, as semicat/net/duo.py:45-55 does
+// through flash_attn's non-interleaved apply_rotary_emb_torch).  The rotation is linear, so tangents
+// take the same rotation as their primals and cotangents the inverse (= transposed) one.
+// Rotate eight column pairs: x0 holds columns j .. j+7 (j = 8 * chunk), x1 columns 32+j .. 32+j+7 of a
+// row at position pos.  sign = +1: y0 = x0 c - x1 s, y1 = x1 c + x0 s; sign = -1: the inverse.
+// fp32 arithmetic, one rounding per element.
+template <typename T>
+__device__ __forceinline__ void rope8(u32x4& x0, u32x4& x1, const RopeTables& rt, int pos, int chunk, float sign) {
+    pos = pos < rt.rows ? pos : rt.rows - 1;
+    const float* cr = rt.cos + (int64_t)pos * rt.cs + 8 * chunk;
+    const float* sr = rt.sin + (int64_t)pos * rt.cs + 8 * chunk;
+    const f32x4 c0 = *reinterpret_cast<const f32x4*>(cr), c1 = *reinterpret_cast<const f32x4*>(cr + 4);
+    const f32x4 s0 = *reinterpret_cast<const f32x4*>(sr), s1 = *reinterpret_cast<const f32x4*>(sr + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float ca = i < 2 ? c0[2 * i] : c1[2 * i - 4], cb = i < 2 ? c0[2 * i + 1] : c1[2 * i - 3];
+        const float sa = sign * (i < 2 ? s0[2 * i] : s1[2 * i - 4]), sb = sign * (i < 2 ? s0[2 * i + 1] : s1[2 * i - 3]);
+        const float a0 = T::to_float((elem_t)(x0[i] & 0xffffu)), a1 = T::to_float((elem_t)(x0[i] >> 16));
+        const float b0 = T::to_float((elem_t)(x1[i] & 0xffffu)), b1 = T::to_float((elem_t)(x1[i] >> 16));
+        x0[i] = T::pack2(fmaf(a0, ca, -b0 * sa), fmaf(a1, cb, -b1 * sb));
+        x1[i] = T::pack2(fmaf(b0, ca, a0 * sa), fmaf(b1, cb, a1 * sb));
+    }
+}
+
+// One output chunk of the inverse rotation from a row held in LDS as 16-byte chunks: chunk c of the
+// result needs chunk c and its partner c ^ 4 of the input (`mine`, `other`).
+template <typename T>
+__device__ __forceinline__ u32x4 rope8_inverse_chunk(u32x4 mine, u32x4 other, const RopeTables& rt, int pos, int c) {
+    u32x4 lo = c < 4 ? mine : other, hi = c < 4 ? other : mine;
+    rope8<T>(lo, hi, rt, pos, c & 3, -1.0f);
+    return c < 4 ? lo : hi;
+}
+
+// Rotate rows of a swizzled [32][64] slab in place: item it (0..127) is row it / 4, chunk pair it % 4.
+template <typename T>
+__device__ __forceinline__ void rope_slab_item(elem_t* slab, int it, const RopeTables& rt, int row0, float sign) {
+    const int r = it >> 2, c = it & 3;
+    u32x4* p0 = reinterpret_cast<u32x4*>(slab + r * 64 + ((c ^ swz<64>(r)) << 3));
+    u32x4* p1 = reinterpret_cast<u32x4*>(slab + r * 64 + (((c + 4) ^ swz<64>(r)) << 3));
+    u32x4 x0 = *p0, x1 = *p1;
+    rope8<T>(x0, x1, rt, row0 + r, c, sign);
+    *p0 = x0;
+    *p1 = x1;
+}
+
 // Per-wave staging tile of the coalesced row stores: [16 rows][HD + 8] elements.
 template <int HD>
 struct StoreStage16 {
@@ -197,9 +244,10 @@ struct StoreStage16 {
 // registers = 4 consecutive columns 16*dt + 4g ..) scaled by mul: 8-byte writes into the wave's
 // staging tile, 16-byte reads back row-major, 16-byte global stores (a 128-byte row per 8 lanes).
 // Issues exactly max(1, HD / 32) global store instructions.
-template <typename T, int HD>
+template <typename T, int HD, bool ROPE = false>
 __device__ __forceinline__ void store_tile16(elem_t* stage, elem_t* gp, int64_t sl, int row0, int L, int D,
-                                             const f32x4* acc, float mul, int lane) {
+                                             const f32x4* acc, float mul, int lane,
+                                             const RopeTables* rt = nullptr) {
     constexpr int P = StoreStage16<HD>::pitch;
     const int n = lane & 15, g = lane >> 4;
 #pragma unroll
@@ -214,7 +262,13 @@ __device__ __forceinline__ void store_tile16(elem_t* stage, elem_t* gp, int64_t 
         const int r = it * RPI + lane / CH;
         const int c = lane % CH;
         if (RPI <= 16 || r < 16) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * P + 8 * c);
+            u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * P + 8 * c);
+            if constexpr (ROPE) {
+                // a gradient of a rotated tensor goes back through the inverse rotation
+                static_assert(!ROPE || HD == 64, "the folded rotation covers a head dimension of 64");
+                const u32x4 other = *reinterpret_cast<const u32x4*>(stage + r * P + 8 * (c ^ 4));
+                v = rope8_inverse_chunk<T>(v, other, *rt, row0 + r, c);
+            }
             if (row0 + r < L && 8 * c < D) {
                 u32x4* dst = reinterpret_cast<u32x4*>(gp + (int64_t)(row0 + r) * sl + 8 * c);
                 __builtin_nontemporal_store(v, dst);  // written once, not read again by this launch

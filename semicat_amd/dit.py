@@ -24,7 +24,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor, nn
 
-from .functional import safe_sdpa_jvp
+from .functional import safe_sdpa_jvp, safe_sdpa_jvp_rotary
 from .rotary import apply_rotary
 
 
@@ -117,6 +117,15 @@ class DDiTBlock(nn.Module):
         h = self.norm1(x) * (1.0 + scale_a) + shift_a
         qkv = self.attn_qkv(h).view(B, self.seq_len, 3, self.n_heads, self.dim // self.n_heads)
         v = qkv[:, :, 2]
+        if rotary_kernel and attention is safe_sdpa_jvp:
+            # the attention kernels read q, k, v (and their tangents) as strided views of the fused
+            # projection and rotate q, k on chip; gradients come back through the inverse rotation
+            # (shapes the folded rotation does not serve take the rotary kernel first)
+            a = safe_sdpa_jvp_rotary(qkv[:, :, 0], qkv[:, :, 1], v, cos, sin)
+            a = a.reshape(B, self.seq_len, self.dim)
+            x = self.dropout(self.attn_out(a) * gate_a) + x
+            h = self.norm2(x) * (1.0 + scale_m) + shift_m
+            return self.dropout(self.mlp(h) * gate_m) + x
         if rotary_kernel:
             # one launch rotates q and k (and their tangents) out of the fused projection and writes
             # the contiguous 16-bit tensors the attention kernels read

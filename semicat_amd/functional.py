@@ -62,9 +62,10 @@ class SDPABackwardFunction(torch.autograd.Function):
     """Gradients for the cotangent on the primal output (functional.py:171-213)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, o, do, M, arith=None):
+    def forward(ctx, q, k, v, o, do, M, arith=None, cos=None, sin=None):
         dq, dk, dv, _, _, _ = kernels.attention_jvp_backward(
-            q, k, v, None, None, None, o, None, M, None, dO=do, dTO=None, arithmetic=arith)
+            q, k, v, None, None, None, o, None, M, None, dO=do, dTO=None, arithmetic=arith,
+            rope=None if cos is None else (cos, sin))
         return dq, dk, dv
 
     @staticmethod
@@ -152,16 +153,18 @@ class SDPAFusedFunction(torch.autograd.Function):
     unpacked by hand (see ``_sdpa``)."""
 
     @staticmethod
-    def forward(q, k, v, t_q, t_k, t_v, seq_major=False, arith=None):
+    def forward(q, k, v, t_q, t_k, t_v, seq_major=False, arith=None, cos=None, sin=None):
         y = _empty_output(q, v.shape[-1], seq_major)
         y, t_y, M, MU, _ = kernels.attention_jvp_forward(q, k, v, t_q, t_k, t_v, o=y, to=torch.empty_like(y),
-                                                         with_li=False, arithmetic=arith)
+                                                         with_li=False, arithmetic=arith,
+                                                         rope=None if cos is None else (cos, sin))
         return y, t_y, M, MU
 
     @staticmethod
     def setup_context(ctx: Any, inputs: tuple[Any, ...], output: Any) -> Any:
         y, t_y, M, MU = output
-        ctx.save_for_backward(*inputs[:6], y, t_y, M, MU)
+        ctx.rope = inputs[8] is not None
+        ctx.save_for_backward(*inputs[:6], y, t_y, M, MU, *(inputs[8:10] if ctx.rope else ()))
         ctx.arith = inputs[7]
         ctx.mark_non_differentiable(M, MU)
         ctx.set_materialize_grads(False)
@@ -169,24 +172,25 @@ class SDPAFusedFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_y, d_t_y, *_):
         if d_y is None and d_t_y is None:
-            return (None,) * 8
-        q, k, v, t_q, t_k, t_v, y, t_y, M, MU = ctx.saved_tensors
+            return (None,) * 10
+        q, k, v, t_q, t_k, t_v, y, t_y, M, MU, *rope = ctx.saved_tensors
+        cos, sin = rope if ctx.rope else (None, None)
         with torch.no_grad():
             if d_t_y is None:
-                dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith)
-                return dq, dk, dv, None, None, None, None, None
+                dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith, cos, sin)
+                return dq, dk, dv, None, None, None, None, None, None, None
             grads = SDPAJVPFusedBackwardFunction.apply(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y,
-                                                       ctx.arith)
-        return *grads, None, None
+                                                       ctx.arith, cos, sin)
+        return *grads, None, None, None, None
 
 
 class SDPAJVPFusedBackwardFunction(torch.autograd.Function):
     """Gradients for cotangents on both outputs in one launch (``d_y`` may be None)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y, arith=None):
+    def forward(ctx, q, k, v, t_q, t_k, t_v, y, t_y, M, MU, d_y, d_t_y, arith=None, cos=None, sin=None):
         return kernels.attention_jvp_backward(q, k, v, t_q, t_k, t_v, y, t_y, M, MU, dO=d_y, dTO=d_t_y,
-                                              arithmetic=arith)
+                                              arithmetic=arith, rope=None if cos is None else (cos, sin))
 
     @staticmethod
     def backward(ctx, *grads):
@@ -197,17 +201,19 @@ class SDPAPrimalFunction(torch.autograd.Function):
     """The op without forward-mode tangents: plain attention with the primal-only kernels."""
 
     @staticmethod
-    def forward(ctx, q, k, v, seq_major=False, arith=None):
-        y, M = kernels.attention_forward(q, k, v, o=_empty_output(q, v.shape[-1], seq_major), arithmetic=arith)
-        ctx.save_for_backward(q, k, v, y, M)
+    def forward(ctx, q, k, v, seq_major=False, arith=None, cos=None, sin=None):
+        rope = None if cos is None else (cos, sin)
+        y, M = kernels.attention_forward(q, k, v, o=_empty_output(q, v.shape[-1], seq_major), arithmetic=arith,
+                                         rope=rope)
+        ctx.save_for_backward(q, k, v, y, M, *(rope or ()))
         ctx.arith = arith
         return y
 
     @staticmethod
     def backward(ctx, d_y):
-        q, k, v, y, M = ctx.saved_tensors
-        dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith)
-        return dq, dk, dv, None, None
+        q, k, v, y, M, *rope = ctx.saved_tensors
+        dq, dk, dv = SDPABackwardFunction.apply(q, k, v, y, d_y, M, ctx.arith, *rope)
+        return dq, dk, dv, None, None, None, None
 
 
 @torch._dynamo.disable
@@ -219,18 +225,21 @@ def sdpa_jvp(q: Tensor, k: Tensor, v: Tensor) -> Tensor:
 
 
 @torch._dynamo.disable
-def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool, arith: Optional[str] = None) -> Tensor:
+def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool, arith: Optional[str] = None,
+          cos: Optional[Tensor] = None, sin: Optional[Tensor] = None) -> Tensor:
     if _has_tangent(q) or _has_tangent(k) or _has_tangent(v):
         if AUTOGRAD_WIRING == "reference":
+            if cos is not None:
+                raise ValueError("the reference wiring has no folded rotary embedding")
             y, _ = SDPAFunction.apply(q, k, v, seq_major)
             return y
         (q, t_q), (k, t_k), (v, t_v) = (fwAD.unpack_dual(t) for t in (q, k, v))
         t_q = torch.zeros_like(q) if t_q is None else t_q
         t_k = torch.zeros_like(k) if t_k is None else t_k
         t_v = torch.zeros_like(v) if t_v is None else t_v
-        y, t_y, _, _ = SDPAFusedFunction.apply(q, k, v, t_q, t_k, t_v, seq_major, arith)
+        y, t_y, _, _ = SDPAFusedFunction.apply(q, k, v, t_q, t_k, t_v, seq_major, arith, cos, sin)
         return fwAD.make_dual(y, t_y)
-    return SDPAPrimalFunction.apply(q, k, v, seq_major, arith)
+    return SDPAPrimalFunction.apply(q, k, v, seq_major, arith, cos, sin)
 
 
 def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Tensor:
@@ -255,3 +264,23 @@ def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Ten
     if y.dtype != orig_dtype:
         y = y.to(orig_dtype)
     return y
+
+
+@torch._dynamo.disable
+def safe_sdpa_jvp_rotary(q: Tensor, k: Tensor, v: Tensor, cos: Tensor, sin: Tensor) -> Tensor:
+    """``safe_sdpa_jvp(rot(q), rot(k), v)`` for ``[B,S,H,D]`` tensors (views of a fused projection are
+    fine), where ``rot`` is the rotary position embedding that semicat/net/duo.py:45-55 applies to q and
+    k in front of the op, with fp32 ``cos``/``sin`` tables ``[S, D/2]``.  Where the kernels serve the
+    shape (head dimension 64, at most 128 keys, bf16 / fp16 inputs with aligned rows) the rotation is
+    folded into the attention launches: q and k are read unrotated, rotated on chip, and the gradients
+    come back through the inverse rotation, so no rotary launch and no rotated copy of q, k exists in
+    either AD mode.  Other shapes rotate with the library's rotary kernel first."""
+    qh, kh, vh = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    tangents = [fwAD.unpack_dual(t).tangent for t in (qh, kh, vh)]
+    if AUTOGRAD_WIRING != "reference" and kernels.rotary_fusable(
+            fwAD.unpack_dual(qh).primal, fwAD.unpack_dual(kh).primal, cos,
+            [fwAD.unpack_dual(vh).primal, *tangents]):
+        return _sdpa(qh, kh, vh, seq_major=True, cos=cos, sin=sin).transpose(1, 2)
+    from .rotary import apply_rotary
+    q, k = apply_rotary((q, k), cos, sin)
+    return safe_sdpa_jvp(q, k, v)

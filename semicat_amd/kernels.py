@@ -36,6 +36,36 @@ def _scale_arg(scale: Optional[float]) -> float:
     return scale
 
 
+def _rope_args(rope, Lq: int, Lk: int, device):
+    """(cos ptr, sin ptr, row stride, rows) of the fp32 ``[rows, 32]`` tables of a folded rotation."""
+    cos, sin = rope
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.ndim != 2 \
+            or cos.shape[1] != 32 or cos.stride(1) != 1 or sin.stride(1) != 1 or cos.stride(0) != sin.stride(0) \
+            or cos.device != device or sin.device != device or cos.shape[0] < max(Lq, Lk):
+        raise AssertionError("folded rotary embedding: cos/sin must be float32 [>= max(Lq, Lk), 32] tensors on "
+                             "the inputs' device with unit column stride and equal row strides")
+    return _ptr(cos), _ptr(sin), cos.stride(0), cos.shape[0]
+
+
+def rotary_fusable(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, others: Sequence[torch.Tensor] = ()) -> bool:
+    """Whether ``[B,H,L,D]`` views q, k (and ``others``: v, tangents) can take the attention kernels
+    with the rotary embedding folded in: head dimension 64 rotated as a whole, at most 128 keys,
+    16-bit tensors with 16-byte aligned rows, 16-byte aligned fp32 tables."""
+    if not q.is_cuda or q.dtype not in (torch.bfloat16, torch.float16) or q.shape[-1] != 64 or k.shape[-2] > 128:
+        return False
+    # Alignment is judged from the offset into the storage (allocations start on 256-byte boundaries):
+    # under torch.func transforms the tensors are wrappers without an address of their own.
+    if cos.shape[-1] != 32 or cos.dtype != torch.float32 or cos.stride(0) % 4 or cos.stride(1) != 1 \
+            or (cos.storage_offset() * 4) % 16:
+        return False
+    for t in (q, k, *others):
+        if t is None:
+            continue
+        if t.dtype != q.dtype or t.stride(-1) != 1 or (t.storage_offset() * 2) % 16 or any(s % 8 for s in t.stride()[:3]):
+            return False
+    return True
+
+
 def stat_rows(L: int) -> int:
     """Length of the row-statistic buffers: L rounded up to 128 (ryu_triton.py:351)."""
     return ((L + 127) // 128) * 128
@@ -106,11 +136,13 @@ def _stat(buf: Optional[torch.Tensor], name: str, B: int, H: int, Lr: int, devic
 
 def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=None, to=None,
                           lse=None, mu=None, li=None, with_li: bool = True, arithmetic: Optional[str] = None,
-                          _plan: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                          rope=None, _plan: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                      Optional[torch.Tensor]]:
     """Fused forward on [B,H,L,D] views: returns (o, to, lse, mu, li); any of them may be passed in
     to be filled in place.  ``with_li=False`` skips the LI statistic (returned as None).
-    ``arithmetic="bf16"`` on float32 tensors: see :func:`_require_gpu`."""
+    ``arithmetic="bf16"`` on float32 tensors: see :func:`_require_gpu`.  ``rope=(cos, sin)``: q, k, tq,
+    tk are given unrotated and the kernel applies the rotary embedding as it loads them
+    (``sjvp_fwd_rotary``; see :func:`rotary_fusable` for the shapes this serves)."""
     dtype_tag = _require_gpu(q, arithmetic)
     B, H, Lq, D = q.shape
     Lk = k.shape[-2]
@@ -138,17 +170,23 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale: Optional[float] = None, o=
         stream = torch.cuda.current_stream().cuda_stream
         args = (_ptr(q), _ptr(k), _ptr(v), _ptr(tq), _ptr(tk), _ptr(tv), _ptr(o), _ptr(to),
                 _ptr(lse), _ptr(mu), _ptr(li), B, H, Lq, Lk, D, _strides((q, k, v, tq, tk, tv, o, to)),
-                _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
+                _scale_arg(scale), dtype_tag)
+        fn = lib.sjvp_fwd
+        if rope is not None:
+            args += _rope_args(rope, Lq, Lk, dev)
+            fn = lib.sjvp_fwd_rotary
+        args += (ctypes.c_void_p(stream),)
         if _plan:
-            return _Launch(lib.sjvp_fwd, args, (q, k, v, tq, tk, tv, o, to, lse, mu, li)), (o, to, lse, mu, li)
-        rc = lib.sjvp_fwd(*args)
+            return _Launch(fn, args, (q, k, v, tq, tk, tv, o, to, lse, mu, li, rope)), (o, to, lse, mu, li)
+        rc = fn(*args)
     _lib.check(rc)
     return o, to, lse, mu, li
 
 
 def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None,
-                      arithmetic: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Primal-only forward (tangent contractions compiled out): returns (o, lse)."""
+                      arithmetic: Optional[str] = None, rope=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Primal-only forward (tangent contractions compiled out): returns (o, lse).  ``rope``: as in
+    :func:`attention_jvp_forward`."""
     dtype_tag = _require_gpu(q, arithmetic)
     B, H, Lq, D = q.shape
     Lk = k.shape[-2]
@@ -167,9 +205,13 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None,
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib.sjvp_fwd(_ptr(q), _ptr(k), _ptr(v), None, None, None, _ptr(o), None, _ptr(lse), None,
-                          None, B, H, Lq, Lk, D, _strides((q, k, v, None, None, None, o, None)),
-                          _scale_arg(scale), dtype_tag, ctypes.c_void_p(stream))
+        args = (_ptr(q), _ptr(k), _ptr(v), None, None, None, _ptr(o), None, _ptr(lse), None,
+                None, B, H, Lq, Lk, D, _strides((q, k, v, None, None, None, o, None)),
+                _scale_arg(scale), dtype_tag)
+        if rope is not None:
+            rc = lib.sjvp_fwd_rotary(*args, *_rope_args(rope, Lq, Lk, dev), ctypes.c_void_p(stream))
+        else:
+            rc = lib.sjvp_fwd(*args, ctypes.c_void_p(stream))
     _lib.check(rc)
     return o, lse
 
@@ -177,7 +219,7 @@ def attention_forward(q, k, v, scale: Optional[float] = None, o=None, lse=None,
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None,
                            scale: Optional[float] = None, grads=None, workspace=None,
                            parts: int = _lib.SJVP_BWD_ALL, static_scratch: bool = False,
-                           arithmetic: Optional[str] = None, _plan: bool = False):
+                           arithmetic: Optional[str] = None, rope=None, _plan: bool = False):
     """Backward on [B,H,L,D] views for cotangents ``dO`` (on o) and ``dTO`` (on to); at least one.
     Returns (dq, dk, dv, dtq, dtk, dtv); the last three are None when ``dTO`` is None (then
     tq, tk, tv, to, mu may be None as well).  ``grads`` optionally supplies the six output buffers
@@ -186,7 +228,9 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
     (profiling only: SJVP_BWD_COL alone needs the workspace an earlier SJVP_BWD_ROW call filled).
     ``static_scratch=True`` takes the ``sjvp_bwd_noalloc`` entry point instead: the workspace is a
     static device array of the library, so with ``grads`` supplied the call allocates nothing; it
-    serves up to ``SJVP_NOALLOC_MAX_ROWS`` statistic rows and calls overlapping on one GPU race."""
+    serves up to ``SJVP_NOALLOC_MAX_ROWS`` statistic rows and calls overlapping on one GPU race.
+    ``rope=(cos, sin)``: q, k, tq, tk are the unrotated tensors the forward was given with the same
+    ``rope``; the gradients returned are those of the unrotated tensors (``sjvp_bwd_rotary``)."""
     dtype_tag = _require_gpu(q, arithmetic)
     if dO is None and dTO is None:
         raise ValueError("attention_jvp_backward needs a cotangent on o, on to, or on both")
@@ -241,6 +285,17 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         return dq, dk, dv, dtq, dtk, dtv
     lib = _lib.load()
     tensors = (q, k, v, tq, tk, tv, o, to, dO, dTO, dq, dk, dv, dtq, dtk, dtv)
+    if rope is not None:
+        if workspace is not None or parts != _lib.SJVP_BWD_ALL or _plan or static_scratch:
+            raise ValueError("rope excludes workspace, parts, static_scratch and planned launches")
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = lib.sjvp_bwd_rotary(*(_ptr(t) for t in tensors[:10]), _ptr(lse), _ptr(mu),
+                                     *(_ptr(t) for t in tensors[10:]), B, H, Lq, Lk, D, _strides(tensors),
+                                     _scale_arg(scale), dtype_tag, *_rope_args(rope, Lq, Lk, dev),
+                                     ctypes.c_void_p(stream))
+        _lib.check(rc)
+        return dq, dk, dv, dtq, dtk, dtv
     if static_scratch:
         if workspace is not None or parts != _lib.SJVP_BWD_ALL or _plan:
             raise ValueError("static_scratch excludes workspace, parts and planned launches")

@@ -26,10 +26,23 @@ def _reader(arithmetic):
     return lambda t: None if t is None else t.detach().float()
 
 
+def _rot(x, rope, inverse=False):
+    """Rotary embedding of a [B,H,L,D] tensor by (cos, sin) [L, D/2] tables; x unchanged without rope."""
+    if rope is None or x is None:
+        return x
+    cos, sin = (t[: x.shape[-2]].float() for t in rope)
+    if inverse:
+        sin = -sin
+    half = cos.shape[-1]
+    x1, x2 = x[..., :half], x[..., half:2 * half]
+    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., 2 * half:]), dim=-1)
+
+
 def attention_jvp_forward(q, k, v, tq, tk, tv, scale=None, o=None, to=None, lse=None, mu=None,
-                          li=None, with_li=True, arithmetic=None):
+                          li=None, with_li=True, arithmetic=None, rope=None):
     f = _reader(arithmetic)
     qf, kf, vf, tqf, tkf, tvf = map(f, (q, k, v, tq, tk, tv))
+    qf, kf, tqf, tkf = (_rot(t, rope) for t in (qf, kf, tqf, tkf))
     s = scale or 1.0 / math.sqrt(q.shape[-1])
     S = s * qf @ kf.transpose(-1, -2)
     TS = s * (tqf @ kf.transpose(-1, -2) + qf @ tkf.transpose(-1, -2))
@@ -54,10 +67,10 @@ def attention_jvp_forward(q, k, v, tq, tk, tv, scale=None, o=None, to=None, lse=
     return o, to, lse, mu, None
 
 
-def attention_forward(q, k, v, scale=None, o=None, lse=None, arithmetic=None):
+def attention_forward(q, k, v, scale=None, o=None, lse=None, arithmetic=None, rope=None):
     f = _reader(arithmetic)
     s = scale or 1.0 / math.sqrt(q.shape[-1])
-    S = s * f(q) @ f(k).transpose(-1, -2)
+    S = s * _rot(f(q), rope) @ _rot(f(k), rope).transpose(-1, -2)
     O = torch.softmax(S, -1) @ f(v)
     lse_, _ = _stats(S, None, q.shape[-2], k.shape[-2])
     o = torch.empty_like(q) if o is None else o
@@ -70,12 +83,12 @@ def attention_forward(q, k, v, scale=None, o=None, lse=None, arithmetic=None):
 
 
 def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=None, scale=None,
-                           grads=None, arithmetic=None):
+                           grads=None, arithmetic=None, rope=None):
     assert dO is not None or dTO is not None
     f = _reader(arithmetic)
     Lq = q.shape[-2]
     s = scale or 1.0 / math.sqrt(q.shape[-1])
-    qf, kf, vf, of = f(q), f(k), f(v), f(o)
+    qf, kf, vf, of = _rot(f(q), rope), _rot(f(k), rope), f(v), f(o)
     T = lambda x: x.transpose(-1, -2)
     P = torch.exp(s * qf @ T(kf) - lse[..., :Lq, None])
     z = torch.zeros_like(of)
@@ -84,7 +97,7 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         dS = P * (dOf @ T(vf) - (dOf * of).sum(-1, keepdim=True))
         out = (s * dS @ kf, s * T(dS) @ qf, T(P) @ dOf, None, None, None)
     else:
-        tqf, tkf, tvf, tof, G = f(tq), f(tk), f(tv), f(to), f(dTO)
+        tqf, tkf, tvf, tof, G = _rot(f(tq), rope), _rot(f(tk), rope), f(tv), f(to), f(dTO)
         N = s * (tqf @ T(kf) + qf @ T(tkf)) - mu[..., :Lq, None]
         s4 = (G * of).sum(-1, keepdim=True)
         s7d = (G * tof).sum(-1, keepdim=True) + (dOf * of).sum(-1, keepdim=True)
@@ -92,6 +105,8 @@ def attention_jvp_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=None, dTO=Non
         dS = dTS * N + P * (G @ T(tvf) + dOf @ T(vf) - s7d)
         out = (s * (dS @ kf + dTS @ tkf), s * (T(dS) @ qf + T(dTS) @ tqf), T(P * N) @ G + T(P) @ dOf,
                s * dTS @ kf, s * T(dTS) @ qf, T(P) @ G)
+    # gradients of rotated tensors go back through the inverse rotation
+    out = tuple(_rot(g, rope, inverse=True) if i in (0, 1, 3, 4) else g for i, g in enumerate(out))
     if grads is None:
         like = (q, k, v, tq, tk, tv)
         return tuple(None if g is None else g.to(l.dtype) for g, l in zip(out, like))

@@ -167,6 +167,17 @@ def test_self_distillation_step_through_the_op_cpu(monkeypatch):
     _compare_steps(net, "cpu", autocast=False, loss_tol=2e-2, grad_tol=8e-2)
 
 
+def test_step_with_the_rotation_folded_into_the_op_cpu(monkeypatch):
+    """The network hands q, k unrotated to safe_sdpa_jvp_rotary; with the launchers replaced by eager
+    stand-ins that apply the rotation themselves (and the inverse rotation to the gradients), losses
+    and gradients equal those of eager math attention behind the PyTorch rotary."""
+    from semicat_amd import kernels
+    eager_backend.install(monkeypatch)
+    monkeypatch.setattr(kernels, "rotary_fusable", lambda *a, **kw: True)
+    net = make_net(rotary="hip")
+    _compare_steps(net, "cpu", autocast=False, loss_tol=2e-2, grad_tol=8e-2)
+
+
 @pytest.mark.gpu
 def test_self_distillation_step_through_the_op_gpu():
     """As above with the HIP kernels, under bf16 autocast as in the reference's training configuration
