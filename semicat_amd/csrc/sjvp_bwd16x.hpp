@@ -412,4 +412,220 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Column-owned kernel for the head dimension 128: a workgroup of eight waves owns 64 keys; waves
+// 2 r and 2 r + 1 share keys 16 r .. 16 r + 15.  Four gradients of 16 x 128 do not fit one wave's
+// registers beside the operands, so the pair splits the work without repeating any of it: member m
+// forms the score-side tiles (S, S_dot, W, XY -> P, P_dot, dS_dot, dS) of the stage's query tile m
+// (16 queries), the two exchange their packed tiles through LDS, and member m accumulates all four
+// gradients for head-dimension columns 64 m .. 64 m + 63 over the stage's 32 queries.  One launch,
+// 12 tile contractions (6 + 6), the query side streamed once.
+// LDS: [ring of Q | [Q_dot | G] | [dO] | lse2, mu, s4, s7d stages][exchange: 8 waves x 4 tiles][sink];
+// the ring doubles as store staging after the last stage.
+template <int HD, int R, bool HAS_DO, bool HAS_G>
+struct Col16pSmem {
+    static constexpr int nt = 1 + (HAS_G ? 2 : 0) + (HAS_DO ? 1 : 0);
+    static constexpr int stat_elems = 4 * kStageRows * 2;
+    static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
+    static constexpr int xch = kWaves16 * 4 * 64 * 4;  // u32x2 per lane, tile and wave, in elem_t units
+    static constexpr int sink = (R * slot + xch) * (int)sizeof(elem_t);
+    static constexpr int bytes = sink + kSink16;
+    static_assert(R * slot >= kWaves16 * StoreStage16<64>::elems, "ring too small to stage stores");
+};
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G>
+__global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdParams p) {
+    static_assert(HD == 128, "the paired form exists for the head dimension that needs it");
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    using SM = Col16pSmem<HD, R, HAS_DO, HAS_G>;
+    elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
+    u32x2* xch = reinterpret_cast<u32x2*>(ring + R * SM::slot);  // [wave][tile 0..3][lane]
+    constexpr int SE = Slab<HD>::elems;
+    constexpr int oTQ = SE, oG = 2 * SE, oDO = (HAS_G ? 3 : 1) * SE, oST = SM::nt * SE;
+    constexpr int KC = HD / 32;
+    constexpr int DH = HD / 32;  // 16-wide head-dimension tiles per member (half of HD / 16)
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int pr = wave >> 1, m = wave & 1;  // pair, member
+    const int n = lane & 15;
+    const int g = lane >> 4;
+    const int k_blocks = (p.Lk + kXOwned16 - 1) / kXOwned16;
+    const int bid = xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
+    const int bh = bid / k_blocks;
+    const int kb = bid % k_blocks;
+    const int b = bh / p.H, h = bh % p.H;
+    const int key0 = kb * kXOwned16;
+    const int krow = key0 + pr * 16 + n;
+    const bool kvalid = krow < p.Lk;
+    const bool pair_active = (key0 + pr * 16) < p.Lk;
+
+    using StagePlan = CopyPlan<HD, SM::nt, 1, kThreads16>;
+    constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics (or its placeholder)
+    StagePlan plan;
+    {
+        const Src q{p.q.head(b, h), p.q.sl};
+        if constexpr (HAS_G && HAS_DO)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
+        else if constexpr (HAS_G)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl});
+        else
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
+    }
+    const int ns = (p.Lq + kStageRows - 1) / kStageRows;
+    int issued = 0;
+    auto issue_next = [&]() {
+        elem_t* slot = ring + (issued % R) * SM::slot;
+        const int row0 = issued * kStageRows;
+        plan.issue(slot, p.Lq - row0);
+        // the four statistic arrays of the stage's rows by waves 0..3; the others issue a placeholder
+        if (wave < 4) {
+            const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;
+            float* st = reinterpret_cast<float*>(slot + oST);
+            if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
+        } else {
+            if (lane == 0) dma4(plan.any, plan.sink);
+        }
+        ++issued;
+    };
+    while (issued < R && issued < ns) issue_next();
+
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
+    load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
+    if constexpr (HAS_G) {
+        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
+        load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+    }
+    const float sl2 = p.scale * kLog2e;
+    f32x4 dk[DH], dv[DH], dtk[DH], dtv[DH];
+#pragma unroll
+    for (int t = 0; t < DH; ++t) {
+        dk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dtv[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // packed tiles of this member's query tile: P, P_dot, dS, dS_dot (register j = query 16 m + 4 g + j)
+    u32x2 mine[4];
+    u32x2* my_x = xch + (wave * 4) * 64 + lane;
+    const u32x2* other_x = xch + ((wave ^ 1) * 4) * 64 + lane;
+
+    auto scores = [&](const elem_t* slot) {
+        const elem_t* sQ = slot;
+        const elem_t* sTQ = slot + oTQ;
+        const elem_t* sG = slot + oG;
+        const elem_t* sDO = slot + oDO;
+        const float* sStat = reinterpret_cast<const float*>(slot + oST);
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, ts = {0.f, 0.f, 0.f, 0.f}, w = {0.f, 0.f, 0.f, 0.f}, xy = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            const u32x4 aq = lds_a_rows16<HD>(sQ, m, c, n, g);
+            s = T::mfma16(aq, kB[c], s);
+            if constexpr (HAS_G) {
+                ts = T::mfma16(aq, tkB[c], ts);
+                const u32x4 atq = lds_a_rows16<HD>(sTQ, m, c, n, g);
+                ts = T::mfma16(atq, kB[c], ts);
+                const u32x4 ag = lds_a_rows16<HD>(sG, m, c, n, g);
+                w = T::mfma16(ag, vB[c], w);
+                xy = T::mfma16(ag, tvB[c], xy);
+            }
+            if constexpr (HAS_DO) {
+                const u32x4 ado = lds_a_rows16<HD>(sDO, m, c, n, g);
+                xy = T::mfma16(ado, vB[c], xy);
+            }
+        }
+        // rows beyond Lq are zero rows of Q, Q_dot, G, dO with finite statistics: they contribute nothing
+        const int r0 = 16 * m + 4 * g;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+        const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+        const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+        const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float pj = fast_exp2(fmaf(s[j], sl2, -lse4[j]));
+            s[j] = pj;
+            if constexpr (HAS_G) {
+                const float nn = fmaf(ts[j], p.scale, -mu4[j]);
+                const float dts = pj * (w[j] - s44[j]);
+                w[j] = dts;
+                xy[j] = fmaf(dts, nn, pj * (xy[j] - s74[j]));
+                ts[j] = pj * nn;
+            } else {
+                xy[j] = pj * (xy[j] - s74[j]);
+            }
+        }
+        mine[0] = u32x2{T::pack2(s[0], s[1]), T::pack2(s[2], s[3])};
+        mine[2] = u32x2{T::pack2(xy[0], xy[1]), T::pack2(xy[2], xy[3])};
+        my_x[0 * 64] = mine[0];
+        my_x[2 * 64] = mine[2];
+        if constexpr (HAS_G) {
+            mine[1] = u32x2{T::pack2(ts[0], ts[1]), T::pack2(ts[2], ts[3])};
+            mine[3] = u32x2{T::pack2(w[0], w[1]), T::pack2(w[2], w[3])};
+            my_x[1 * 64] = mine[1];
+            my_x[3 * 64] = mine[3];
+        }
+    };
+    // B operand over the stage's 32 queries from the pair's two packed tiles (query tile 0 first)
+    auto both = [&](int which) {
+        const u32x2 o = other_x[which * 64];
+        return m == 0 ? u32x4{mine[which][0], mine[which][1], o[0], o[1]}
+                      : u32x4{o[0], o[1], mine[which][0], mine[which][1]};
+    };
+    auto outputs = [&](const elem_t* slot) {
+        const elem_t* sQ = slot;
+        const elem_t* sTQ = slot + oTQ;
+        const elem_t* sG = slot + oG;
+        const elem_t* sDO = slot + oDO;
+        const u32x4 pB = both(0), dsB = both(2);
+        u32x4 pdB, dtsB;
+        if constexpr (HAS_G) {
+            pdB = both(1);
+            dtsB = both(3);
+        }
+#pragma unroll
+        for (int d = 0; d < DH; ++d) {
+            const int d0 = 64 * m + 16 * d;
+            const u32x4 aq = lds_a_tr16<HD>(sQ, d0, lane);
+            dk[d] = T::mfma16(aq, dsB, dk[d]);
+            if constexpr (HAS_G) {
+                dtk[d] = T::mfma16(aq, dtsB, dtk[d]);
+                const u32x4 atq = lds_a_tr16<HD>(sTQ, d0, lane);
+                dk[d] = T::mfma16(atq, dtsB, dk[d]);
+                const u32x4 ag = lds_a_tr16<HD>(sG, d0, lane);
+                dtv[d] = T::mfma16(ag, pB, dtv[d]);
+                dv[d] = T::mfma16(ag, pdB, dv[d]);
+            }
+            if constexpr (HAS_DO) {
+                const u32x4 ado = lds_a_tr16<HD>(sDO, d0, lane);
+                dv[d] = T::mfma16(ado, pB, dv[d]);
+            }
+        }
+    };
+
+    for (int i = 0; i < ns; ++i) {
+        wait_stages<SPT>(issued - 1 - i);
+        __syncthreads();  // stage i has landed for every wave; stage i-1 and the exchange area are free
+        if (i > 0 && issued < ns) issue_next();
+        const elem_t* slot = ring + (i % R) * SM::slot;
+        if (pair_active) scores(slot);
+        __syncthreads();  // the partner's tiles are visible
+        if (pair_active) outputs(slot);
+    }
+    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    if (!pair_active) return;
+    elem_t* stage_tile = ring + wave * StoreStage16<64>::elems;
+    const int row0 = key0 + pr * 16;
+    const int dcol = 64 * m;
+    const int Dm = p.D - dcol;  // columns of this member's half that exist (may be <= 0)
+    store_tile16<T, 64>(stage_tile, p.dk.head(b, h) + dcol, p.dk.sl, row0, p.Lk, Dm, dk, p.scale, lane);
+    if constexpr (HAS_G)
+        store_tile16<T, 64>(stage_tile, p.dtk.head(b, h) + dcol, p.dtk.sl, row0, p.Lk, Dm, dtk, p.scale, lane);
+    store_tile16<T, 64>(stage_tile, p.dv.head(b, h) + dcol, p.dv.sl, row0, p.Lk, Dm, dv, 1.0f, lane);
+    if constexpr (HAS_G)
+        store_tile16<T, 64>(stage_tile, p.dtv.head(b, h) + dcol, p.dtv.sl, row0, p.Lk, Dm, dtv, 1.0f, lane);
+}
+
 }  // namespace sjvp

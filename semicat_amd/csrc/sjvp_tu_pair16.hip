@@ -2,6 +2,10 @@
 #include "sjvp_bwd16x.hpp"
 #include "sjvp_launch.hpp"
 
+#ifndef SJVP_COL16P_RING
+#define SJVP_COL16P_RING 2
+#endif
+
 namespace sjvp {
 namespace {
 
@@ -18,10 +22,11 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     const int grid = BH * ((p.Lk + kXOwned16 - 1) / kXOwned16);
     using CS = Col16Smem<HD, XR, HAS_DO, HAS_G>;
     if constexpr (HD == 128) {
-        // two launches, each accumulating two of the four gradients (register budget)
-        rc = launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 1, 2>, grid, CS::bytes, stream, p, kXThreads16);
-        if (rc != SJVP_OK) return rc;
-        return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 2, 2>, grid, CS::bytes, stream, p, kXThreads16);
+        // eight waves: wave pairs share 16 keys, split the score-side tiles by query tile and the
+        // gradients by head-dimension half (one launch, nothing computed twice)
+        constexpr int PR = SJVP_COL16P_RING;  // ring depths 2, 3, 4 measure the same (the kernel is issue-bound)
+        return launch(bwd_col16p_kernel<T, HD, PR, HAS_DO, HAS_G>, grid, Col16pSmem<HD, PR, HAS_DO, HAS_G>::bytes,
+                      stream, p, kThreads16);
     } else {
         return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
     }
