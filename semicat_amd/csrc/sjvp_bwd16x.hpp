@@ -304,57 +304,96 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         const elem_t* sG = slot + oG;
         const elem_t* sDO = slot + oDO;
         const float* sStat = reinterpret_cast<const float*>(slot + oST);
-        // tiles: rows = queries (registers), columns = this wave's keys (lanes)
+        // tiles: rows = queries (registers), columns = this wave's keys (lanes).
+        // The A operands of every contraction step are read from LDS one step ahead of the MFMAs
+        // that use them (two register sets), so that a wave's matrix pipe does not sit out an LDS
+        // round trip per step; the first operands of the gradient phase and the row statistics are
+        // requested before the last score step and arrive during the element-wise work.
+        struct AOps {
+            u32x4 q, tq, g, d;
+        };
+        auto load_score = [&](int t, int c) {
+            AOps a;
+            a.q = lds_a_rows16<HD>(sQ, t, c, n, g);
+            if constexpr (HAS_G) {
+                a.tq = lds_a_rows16<HD>(sTQ, t, c, n, g);
+                if constexpr (DO_K) a.g = lds_a_rows16<HD>(sG, t, c, n, g);
+            }
+            if constexpr (HAS_DO && DO_K) a.d = lds_a_rows16<HD>(sDO, t, c, n, g);
+            return a;
+        };
+        auto load_grad = [&](int d) {
+            AOps a;
+            if constexpr (DO_K) {
+                a.q = lds_a_tr16<HD>(sQ, 16 * d, lane);
+                if constexpr (HAS_G) a.tq = lds_a_tr16<HD>(sTQ, 16 * d, lane);
+            }
+            if constexpr (DO_V) {
+                if constexpr (HAS_G) a.g = lds_a_tr16<HD>(sG, 16 * d, lane);
+                if constexpr (HAS_DO) a.d = lds_a_tr16<HD>(sDO, 16 * d, lane);
+            }
+            return a;
+        };
         f32x4 s[2], ts[2], w[2], xy[2];
+        f32x4 lse4[2], mu4[2], s44[2], s74[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        AOps cur = load_score(0, 0);
 #pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                const u32x4 aq = lds_a_rows16<HD>(sQ, t, c, n, g);
-                s[t] = T::mfma16(aq, kB[c], s[t]);
-                if constexpr (HAS_G) {
-                    ts[t] = T::mfma16(aq, tkB[c], ts[t]);
-                    const u32x4 atq = lds_a_rows16<HD>(sTQ, t, c, n, g);
-                    ts[t] = T::mfma16(atq, kB[c], ts[t]);
-                    if constexpr (DO_K) {
-                        const u32x4 ag = lds_a_rows16<HD>(sG, t, c, n, g);
-                        w[t] = T::mfma16(ag, vB[c], w[t]);
-                        xy[t] = T::mfma16(ag, tvB[c], xy[t]);
-                    }
+        for (int j = 0; j < 2 * KC; ++j) {
+            const int t = j / KC, c = j % KC;
+            AOps nxt;
+            if (j + 1 < 2 * KC) {
+                nxt = load_score((j + 1) / KC, (j + 1) % KC);
+            } else {
+                // register j of tile t is query 16 t + 4 g + j
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int r0 = 16 * u + 4 * g;
+                    lse4[u] = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+                    if constexpr (HAS_G) mu4[u] = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+                    if constexpr (HAS_G && DO_K) s44[u] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+                    if constexpr (DO_K) s74[u] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
                 }
-                if constexpr (HAS_DO && DO_K) {
-                    const u32x4 ado = lds_a_rows16<HD>(sDO, t, c, n, g);
-                    xy[t] = T::mfma16(ado, vB[c], xy[t]);
+                nxt = load_grad(0);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of this step's MFMAs
+            s[t] = T::mfma16(cur.q, kB[c], s[t]);
+            if constexpr (HAS_G) {
+                ts[t] = T::mfma16(cur.q, tkB[c], ts[t]);
+                ts[t] = T::mfma16(cur.tq, kB[c], ts[t]);
+                if constexpr (DO_K) {
+                    w[t] = T::mfma16(cur.g, vB[c], w[t]);
+                    xy[t] = T::mfma16(cur.g, tvB[c], xy[t]);
                 }
             }
+            if constexpr (HAS_DO && DO_K) xy[t] = T::mfma16(cur.d, vB[c], xy[t]);
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
         }
-        // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (register j of tile t is query 16t + 4g + j;
-        // rows beyond Lq are zero rows of Q, Q_dot, G, dO with finite statistics: they contribute nothing)
+        // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (rows beyond Lq are zero rows of Q,
+        // Q_dot, G, dO with finite statistics: they contribute nothing)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int r0 = 16 * t + 4 * g;
-            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
-            const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
-            const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
-            const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
+                const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[t][j]));
                 s[t][j] = pj;
                 if constexpr (HAS_G) {
-                    const float nn = fmaf(ts[t][j], p.scale, -mu4[j]);
+                    const float nn = fmaf(ts[t][j], p.scale, -mu4[t][j]);
                     if constexpr (DO_K) {
-                        const float dts = pj * (w[t][j] - s44[j]);
+                        const float dts = pj * (w[t][j] - s44[t][j]);
                         w[t][j] = dts;
-                        xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[j]));
+                        xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[t][j]));
                     }
                     if constexpr (DO_V) ts[t][j] = pj * nn;
                 } else if constexpr (DO_K) {
-                    xy[t][j] = pj * (xy[t][j] - s74[j]);
+                    xy[t][j] = pj * (xy[t][j] - s74[t][j]);
                 }
             }
         }
@@ -367,26 +406,25 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         }
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
+            AOps nxt;
+            if (d + 1 < DT) nxt = load_grad(d + 1);
+            __builtin_amdgcn_sched_barrier(0);
             if constexpr (DO_K) {
-                const u32x4 aq = lds_a_tr16<HD>(sQ, 16 * d, lane);
-                dk[d] = T::mfma16(aq, dsB, dk[d]);
+                dk[d] = T::mfma16(cur.q, dsB, dk[d]);
                 if constexpr (HAS_G) {
-                    dtk[d] = T::mfma16(aq, dtsB, dtk[d]);
-                    const u32x4 atq = lds_a_tr16<HD>(sTQ, 16 * d, lane);
-                    dk[d] = T::mfma16(atq, dtsB, dk[d]);
+                    dtk[d] = T::mfma16(cur.q, dtsB, dtk[d]);
+                    dk[d] = T::mfma16(cur.tq, dtsB, dk[d]);
                 }
             }
             if constexpr (DO_V) {
                 if constexpr (HAS_G) {
-                    const u32x4 ag = lds_a_tr16<HD>(sG, 16 * d, lane);
-                    dtv[d] = T::mfma16(ag, pB, dtv[d]);
-                    dv[d] = T::mfma16(ag, pdB, dv[d]);
+                    dtv[d] = T::mfma16(cur.g, pB, dtv[d]);
+                    dv[d] = T::mfma16(cur.g, pdB, dv[d]);
                 }
-                if constexpr (HAS_DO) {
-                    const u32x4 ado = lds_a_tr16<HD>(sDO, 16 * d, lane);
-                    dv[d] = T::mfma16(ado, pB, dv[d]);
-                }
+                if constexpr (HAS_DO) dv[d] = T::mfma16(cur.d, pB, dv[d]);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
         }
     };
 

@@ -205,20 +205,28 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         }
     };
 
-    for (int i = 0; i < ns; i += SPB) {
-        if (i > 0) {
-            // the stages of this step have landed for every wave; those of the last step are consumed
-            wait_stages<SPT>(SPB == 2 ? 0 : issued - 1 - i);
-            __syncthreads();
+    // One trip of the outer loop goes once round the ring, so that every LDS address of the
+    // unrolled body is a per-lane constant plus an immediate offset.
+    static_assert(R % SPB == 0, "a step must not wrap the ring");
+    for (int i0 = 0; i0 < ns; i0 += R) {
+#pragma unroll
+        for (int h = 0; h < R; h += SPB) {
+            const int i = i0 + h;
+            if (i >= ns) break;
+            if (i > 0) {
+                // the stages of this step have landed for every wave; those of the last step are consumed
+                wait_stages<SPT>(SPB == 2 ? 0 : issued - 1 - i);
+                __syncthreads();
+#pragma unroll
+                for (int u = 0; u < SPB; ++u)
+                    if (issued < ns) issue_next();
+                rotate_stage(ring + h * SM::slot, i * kStageRows);
+            }
+            if (!wave_active) continue;
 #pragma unroll
             for (int u = 0; u < SPB; ++u)
-                if (issued < ns) issue_next();
-            rotate_stage(ring + (i % R) * SM::slot, i * kStageRows);
+                if (i + u < ns) compute(ring + (h + u) * SM::slot, (i + u) * kStageRows);
         }
-        if (!wave_active) continue;
-#pragma unroll
-        for (int u = 0; u < SPB; ++u)
-            if (i + u < ns) compute(ring + ((i + u) % R) * SM::slot, (i + u) * kStageRows);
     }
     __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
     const int64_t so = (int64_t)bh * p.Lr + qrow;
