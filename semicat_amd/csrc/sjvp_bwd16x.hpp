@@ -343,43 +343,28 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
             w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        AOps cur = load_score(0, 0);
-#pragma unroll
-        for (int j = 0; j < 2 * KC; ++j) {
-            const int t = j / KC, c = j % KC;
-            AOps nxt;
-            if (j + 1 < 2 * KC) {
-                nxt = load_score((j + 1) / KC, (j + 1) % KC);
-            } else {
-                // register j of tile t is query 16 t + 4 g + j
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const int r0 = 16 * u + 4 * g;
-                    lse4[u] = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
-                    if constexpr (HAS_G) mu4[u] = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
-                    if constexpr (HAS_G && DO_K) s44[u] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
-                    if constexpr (DO_K) s74[u] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
-                }
-                nxt = load_grad(0);
-            }
-            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of this step's MFMAs
-            s[t] = T::mfma16(cur.q, kB[c], s[t]);
+        auto load_stats = [&](int u) __attribute__((always_inline)) {
+            const int r0 = 16 * u + 4 * g;  // register j of tile u is query 16 u + 4 g + j
+            lse4[u] = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
+            if constexpr (HAS_G) mu4[u] = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
+            if constexpr (HAS_G && DO_K) s44[u] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+            if constexpr (DO_K) s74[u] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+        };
+        auto score_step = [&](int t, int c, const AOps& a) __attribute__((always_inline)) {
+            s[t] = T::mfma16(a.q, kB[c], s[t]);
             if constexpr (HAS_G) {
-                ts[t] = T::mfma16(cur.q, tkB[c], ts[t]);
-                ts[t] = T::mfma16(cur.tq, kB[c], ts[t]);
+                ts[t] = T::mfma16(a.q, tkB[c], ts[t]);
+                ts[t] = T::mfma16(a.tq, kB[c], ts[t]);
                 if constexpr (DO_K) {
-                    w[t] = T::mfma16(cur.g, vB[c], w[t]);
-                    xy[t] = T::mfma16(cur.g, tvB[c], xy[t]);
+                    w[t] = T::mfma16(a.g, vB[c], w[t]);
+                    xy[t] = T::mfma16(a.g, tvB[c], xy[t]);
                 }
             }
-            if constexpr (HAS_DO && DO_K) xy[t] = T::mfma16(cur.d, vB[c], xy[t]);
-            __builtin_amdgcn_sched_barrier(0);
-            cur = nxt;
-        }
+            if constexpr (HAS_DO && DO_K) xy[t] = T::mfma16(a.d, vB[c], xy[t]);
+        };
         // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (rows beyond Lq are zero rows of Q,
         // Q_dot, G, dO with finite statistics: they contribute nothing)
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        auto pointwise = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[t][j]));
@@ -396,7 +381,33 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
                     xy[t][j] = pj * (xy[t][j] - s74[t][j]);
                 }
             }
+        };
+        AOps cur = load_score(0, 0);
+        load_stats(0);
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            AOps nxt = c + 1 < KC ? load_score(0, c + 1) : load_score(1, 0);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of this step's MFMAs
+            score_step(0, c, cur);
+            __builtin_amdgcn_sched_barrier(0);
+            cur = nxt;
         }
+        // the second tile's MFMA chains run under the first tile's element-wise arithmetic
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            AOps nxt;
+            if (c + 1 < KC) {
+                nxt = load_score(1, c + 1);
+            } else {
+                load_stats(1);
+                nxt = load_grad(0);
+            }
+            score_step(1, c, cur);
+            cur = nxt;
+        }
+        pointwise(0);
+        __builtin_amdgcn_sched_barrier(0);
+        pointwise(1);
         u32x4 pB, dsB, pdB, dtsB;
         if constexpr (DO_V) pB = pack_b16<T>(s[0], s[1]);
         if constexpr (DO_K) dsB = pack_b16<T>(xy[0], xy[1]);
