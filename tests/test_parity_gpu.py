@@ -620,6 +620,59 @@ def test_randomized_shapes_layouts_and_modes(K):
     print(f"worst relative error over the sweep: {worst:.2e}")
 
 
+def test_randomized_shapes_on_the_fp32_kernels_and_the_folded_casts(K):
+    """The seeded sweep of test_randomized_shapes_layouts_and_modes on fp32 tensors: the fp32 kernels
+    (every head-dimension class, odd head dimensions, lengths around their 16-row tiles and 32-row
+    blocks) at 1e-5 against the fp64 oracle, and arithmetic="bf16" (casts folded into loads and stores;
+    both 16-bit kernel families) at the 16-bit gate against the oracle on the rounded inputs."""
+    import random
+    rng = random.Random(4321)
+    worst = {"fp32": 0.0, "bf16": 0.0}
+    for case in range(48):
+        arith = "bf16" if case % 2 else None
+        D = rng.choice([16, 20, 32, 40, 48, 64, 64, 100, 128])
+        Lq = rng.choice([1, 15, 16, 17, 31, 32, 33, 64, 100, 127, 128, 129, 200, 257])
+        Lk = rng.choice([1, 3, 15, 16, 17, 31, 32, 33, 64, 96, 127, 128, 129, 255, 257, 300])
+        B, H = rng.choice([1, 2]), rng.choice([1, 2, 3])
+        mode = rng.choice(["both", "both", "dO", "dTO"])
+        seq_major = rng.random() < 0.5
+        label = f"case {case}: B{B} H{H} Lq{Lq} Lk{Lk} D{D} arithmetic={arith} {mode} seq_major={seq_major}"
+        print(label, flush=True)
+        x = orc.make_inputs(B, H, Lq, Lk, D, seed=100 + case, tangent_scale=0.3, dtype=torch.float32)
+        xo = {n: t.to(torch.bfloat16) for n, t in x.items()} if arith else x
+        cot = {}
+        if mode != "dTO":
+            cot["dO"] = xo["dO"]
+        if mode != "dO":
+            cot["dTO"] = xo["dTO"]
+        ref = orc.attention_jvp_autograd(*[xo[n] for n in orc.TENSOR_ORDER[:6]], **cot)
+        d = {n: (t.cuda().transpose(1, 2).contiguous().transpose(1, 2) if seq_major else t.cuda())
+             for n, t in x.items()}
+        kw = {"arithmetic": arith} if arith else {}
+        o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], **kw)
+        if mode == "dO":
+            g = K.attention_jvp_backward(d["q"], d["k"], d["v"], None, None, None, o, None, lse, None,
+                                         dO=d["dO"], **kw)
+        else:
+            g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                         dO=d["dO"] if mode == "both" else None, dTO=d["dTO"], **kw)
+        res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g) if t is not None}}
+        tol = TOL_16BIT if arith else TOL_FP32
+        floor = max(ref[m].double().norm().item() for m in GRADS if ref.get(m) is not None)
+        for n, t in res.items():
+            assert t.dtype == torch.float32 and torch.isfinite(t).all(), (label, n)
+            err = (t.double() - ref[n].double()).norm().item()
+            scale = ref[n].double().norm().item()
+            if Lk == 1 and n in GRADS:
+                scale = max(scale, floor)  # a single key: several gradients vanish identically
+            assert err <= tol * max(scale, 1e-30), (label, n, err / max(scale, 1e-30))
+            worst[arith or "fp32"] = max(worst[arith or "fp32"], err / max(scale, 1e-30))
+        o2, lse2 = K.attention_forward(d["q"], d["k"], d["v"], **kw)
+        assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= tol, label
+        assert torch.allclose(lse2[..., :Lq], lse[..., :Lq], rtol=1e-5, atol=1e-5), label
+    print(f"worst relative error: fp32 kernels {worst['fp32']:.2e}, folded casts {worst['bf16']:.2e}")
+
+
 def test_graph_replays_match_eager_launches(K):
     """The launches are capturable in a HIP graph (no allocation, no memset, no host synchronisation
     inside the library): three replays, with the program's own eager work and synchronisations between
