@@ -1,5 +1,6 @@
 // C ABI of the attention-JVP library (declared in include/sjvp.h): argument validation, kernel
-// selection and launches.  No device memory is allocated or freed here and no state is kept.
+// selection and launches.  No device memory is allocated or freed here; the only state kept is the
+// per-device address of the static scratch array that sjvp_bwd_noalloc() works in.
 #include "../../include/sjvp.h"
 
 #include <hip/hip_runtime.h>
