@@ -673,6 +673,50 @@ def test_randomized_shapes_on_the_fp32_kernels_and_the_folded_casts(K):
     print(f"worst relative error: fp32 kernels {worst['fp32']:.2e}, folded casts {worst['bf16']:.2e}")
 
 
+@pytest.mark.parametrize("L,D,dtype", [(128, 64, torch.bfloat16), (160, 64, torch.bfloat16),
+                                       (100, 20, torch.bfloat16), (70, 64, torch.float32)])
+def test_batch_strides_beyond_32_bits(K, L, D, dtype):
+    """Tensors that are views with a batch stride of more than 2^31 elements (the second batch lies
+    more than 4 GiB into its buffer): offsets are 64-bit throughout.  The results equal, bit for bit,
+    those of the same launches on compact copies: on the single-launch backward (L = 128), the row +
+    column pair (L = 160), the register-staged kernels (D = 20) and the fp32 kernels (there q, k, v, the
+    cotangents and O, dq, dk, dv lie far apart; sixteen 8 GiB buffers would be more than the test needs)."""
+    B, H = 2, 2
+    step = 2 ** 31 + 4096  # elements between the two batches
+    x = orc.make_inputs(B, H, L, L, D, seed=31, tangent_scale=0.3, dtype=dtype)
+    near = {"tq", "tk", "tv"} if dtype == torch.float32 else set()
+
+    def far(t=None, compact=False):
+        if compact:
+            return torch.empty((B, H, L, D), dtype=dtype, device="cuda") if t is None else t.cuda()
+        buf = torch.empty(step + H * L * D, dtype=dtype, device="cuda")  # only two slices are ever touched
+        view = buf.as_strided((B, H, L, D), (step, L * D, D, 1))
+        if t is not None:
+            view.copy_(t)
+        return view
+
+    d = {n: far(t, compact=n in near) for n, t in x.items()}
+    c = {n: t.cuda() for n, t in x.items()}
+    assert d["q"].stride(0) > 2 ** 31
+    o, to = far(), far(compact=bool(near))
+    grads = tuple(far(compact=bool(near) and i >= 3) for i in range(6))
+    _, _, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o=o, to=to)
+    K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                             dO=d["dO"], dTO=d["dTO"], grads=grads)
+    o2, to2, lse2, mu2, _ = K.attention_jvp_forward(c["q"], c["k"], c["v"], c["tq"], c["tk"], c["tv"])
+    g2 = K.attention_jvp_backward(c["q"], c["k"], c["v"], c["tq"], c["tk"], c["tv"], o2, to2, lse2, mu2,
+                                  dO=c["dO"], dTO=c["dTO"])
+    torch.cuda.synchronize()
+    for name, a, b in zip(("O", "TO", "lse", "mu") + GRADS, (o, to, lse, mu) + grads, (o2, to2, lse2, mu2) + tuple(g2)):
+        assert torch.equal(a, b), name
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, grads)}}
+    assert_parity(res, ref, TOL_FP32 if dtype == torch.float32 else TOL_16BIT,
+                  label=f"batch stride 2^31+4096, L={L} D={D} {dtype}")
+    del d, o, to, grads
+    torch.cuda.empty_cache()
+
+
 def test_graph_replays_match_eager_launches(K):
     """The launches are capturable in a HIP graph (no allocation, no memset, no host synchronisation
     inside the library): three replays, with the program's own eager work and synchronisations between
