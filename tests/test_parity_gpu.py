@@ -717,6 +717,82 @@ def test_batch_strides_beyond_32_bits(K, L, D, dtype):
     torch.cuda.empty_cache()
 
 
+def test_sequence_strides_beyond_32_bits(K):
+    """Rows 2^22 elements apart: the last of the 600 rows starts 2.5 G elements into its buffer (q, k and
+    the outputs O, dq; the row + column pair and, with 100 rows, the single-launch backward)."""
+    B, H, D, sl = 1, 1, 64, 2 ** 22
+    for L in (600, 100):
+        x = orc.make_inputs(B, H, L, L, D, seed=37, tangent_scale=0.3, dtype=torch.bfloat16)
+        c = {n: t.cuda() for n, t in x.items()}
+
+        def far(t=None):
+            buf = torch.empty(L * sl, dtype=torch.bfloat16, device="cuda")
+            view = buf.as_strided((B, H, L, D), (L * sl, L * sl, sl, 1))
+            if t is not None:
+                view.copy_(t)
+            return view
+
+        d = dict(c, q=far(x["q"]), k=far(x["k"]))
+        o = far()
+        grads = (far(),) + tuple(torch.empty_like(c["q"]) for _ in range(5))
+        _, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o=o)
+        K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"], grads=grads)
+        o2, to2, lse2, mu2, _ = K.attention_jvp_forward(c["q"], c["k"], c["v"], c["tq"], c["tk"], c["tv"])
+        g2 = K.attention_jvp_backward(c["q"], c["k"], c["v"], c["tq"], c["tk"], c["tv"], o2, to2, lse2, mu2,
+                                      dO=c["dO"], dTO=c["dTO"])
+        torch.cuda.synchronize()
+        for name, a, b in zip(("O", "TO", "lse", "mu") + GRADS, (o, to, lse, mu) + grads,
+                              (o2, to2, lse2, mu2) + tuple(g2)):
+            assert torch.equal(a, b), (L, name)
+        del d, o, grads
+        torch.cuda.empty_cache()
+
+
+def test_many_heads_small_problems(K):
+    """131072 (batch, head) pairs of 16 x 16 x 16: grids far beyond 65535 workgroups, every pair against
+    the fp64 oracle (forward and both-cotangent backward)."""
+    B, H, L, D = 4096, 32, 16, 16
+    x = orc.make_inputs(B, H, L, L, D, seed=41, tangent_scale=0.3, dtype=torch.bfloat16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    res = run_hip(K, x)
+    assert_parity(res, ref, TOL_16BIT, label="131072 heads")
+    # no pair is skipped or written twice: the error per pair is uniformly small
+    per_pair = ((res["dk"].double() - ref["dk"].double()).flatten(2).norm(dim=-1)
+                / ref["dk"].double().flatten(2).norm(dim=-1).clamp_min(1e-30))
+    assert per_pair.max().item() <= 5e-2, per_pair.max().item()
+
+
+def test_concurrent_streams_do_not_interfere(K):
+    """The library keeps no per-call state: forward + backward steps of two different problems issued
+    alternately on two streams (own outputs and workspaces each) give the results of running them
+    alone."""
+    shapes = [(2, 3, 128, 64), (1, 2, 300, 64)]
+    xs = [orc.make_inputs(B, H, L, L, D, seed=43 + i, tangent_scale=0.3, dtype=torch.bfloat16)
+          for i, (B, H, L, D) in enumerate(shapes)]
+    ds = [{n: t.cuda() for n, t in x.items()} for x in xs]
+
+    def step(d):
+        o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+        g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                     dO=d["dO"], dTO=d["dTO"])
+        return (o, to, lse, mu) + tuple(g)
+
+    alone = [step(d) for d in ds]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for _ in range(5):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                outs[i].append(step(ds[i]))
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        for rep in outs[i]:
+            for a, b in zip(rep, alone[i]):
+                assert torch.equal(a, b)
+
+
 def test_graph_replays_match_eager_launches(K):
     """The launches are capturable in a HIP graph (no allocation, no memset, no host synchronisation
     inside the library): three replays, with the program's own eager work and synchronisations between
