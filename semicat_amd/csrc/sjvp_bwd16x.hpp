@@ -139,8 +139,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         const elem_t* sTV = slot + 3 * SE;
         // tiles: rows = keys (registers), columns = this wave's queries (lanes)
         f32x4 s[2], ts[2], w[2], xy[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        auto scores = [&](int t) __attribute__((always_inline)) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -160,10 +159,10 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                 }
                 if constexpr (HAS_DO) xy[t] = T::mfma16(av, doB[c], xy[t]);
             }
-        }
+        };
         const bool ragged = k0 + kStageRows > p.Lk;  // wave-uniform: only the last stage
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        // in place: w -> dS_dot, xy -> dS
+        auto pointwise = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float pj = fast_exp2(fmaf(s[t][j], sl2, -lse2));
@@ -179,19 +178,38 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                     xy[t][j] = pj * (xy[t][j] - s7d);
                 }
             }
-        }
+        };
+        // the second key tile's MFMA chains run under the first tile's element-wise arithmetic
+        scores(0);
+        __builtin_amdgcn_sched_barrier(0);
+        scores(1);
+        pointwise(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // the transposed operands of the output contractions are read one step ahead, the first ones
+        // under the second tile's element-wise arithmetic
+        u32x4 ak = lds_a_tr16<HD>(sK, 0, lane), atk;
+        if constexpr (HAS_G) atk = lds_a_tr16<HD>(sTK, 0, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        pointwise(1);
         const u32x4 dsB = pack_b16<T>(xy[0], xy[1]);
         u32x4 dtsB;
         if constexpr (HAS_G) dtsB = pack_b16<T>(w[0], w[1]);
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
-            const u32x4 ak = lds_a_tr16<HD>(sK, 16 * d, lane);
+            u32x4 nk, ntk;
+            if (d + 1 < DT) {
+                nk = lds_a_tr16<HD>(sK, 16 * (d + 1), lane);
+                if constexpr (HAS_G) ntk = lds_a_tr16<HD>(sTK, 16 * (d + 1), lane);
+            }
+            __builtin_amdgcn_sched_barrier(0);
             dq[d] = T::mfma16(ak, dsB, dq[d]);
             if constexpr (HAS_G) {
                 dtq[d] = T::mfma16(ak, dtsB, dtq[d]);
-                const u32x4 atk = lds_a_tr16<HD>(sTK, 16 * d, lane);
                 dq[d] = T::mfma16(atk, dtsB, dq[d]);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            ak = nk;
+            if constexpr (HAS_G) atk = ntk;
         }
     };
 
