@@ -330,6 +330,40 @@ def reference_rounding_error_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfl
             "dtq": dtq, "dtk": dtk, "dtv": dtv}
 
 
+def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, sums_from_outputs=True,
+                           scale: Optional[float] = None) -> Dict[str, np.ndarray]:
+    """The query-side and key-side gradients with the two row sums of the backward formed either from
+    the outputs rounded to ``dtype`` (``s4 = rowsum(G*O)``, ``s7d = rowsum(G*TO) + rowsum(dO*O)``: the
+    FlashAttention "delta" form, extended to the cotangent on the tangent output) or from the
+    probabilities themselves (``rowsum(P*W)``, ``rowsum(P*(N*W + XY))``, what the reference's preprocess
+    kernel does, flash_jvp_backward.py:2012-2290); everything else exact up to one rounding of the
+    score-gradient tiles and of the results.  ``sum_j P (W - s4) = 0`` holds exactly only in the second
+    form; in the first the rounding of O leaves a residue that is the same for every key of a row and
+    so adds up coherently in ``dS_dot^T Q`` and ``dS_dot K``.  Returns dq, dk, dtq, dtk."""
+    r = lambda x: _round_to(x, dtype)
+    q, k, v, tq, tk, tv, dOn, G = (r(_f64(x).numpy()) for x in (q, k, v, tq, tk, tv, dO, dTO))
+    s = 1.0 / math.sqrt(q.shape[-1]) if scale is None else float(scale)
+    T = lambda x: np.swapaxes(x, -1, -2)
+    S = s * (q @ T(k))
+    E = np.exp(S - S.max(-1, keepdims=True))
+    P = E / E.sum(-1, keepdims=True)
+    TS = s * (tq @ T(k) + q @ T(tk))
+    N = TS - (P * TS).sum(-1, keepdims=True)
+    O, TO = r(P @ v), r((P * N) @ v + P @ tv)
+    W, XY = G @ T(v), G @ T(tv) + dOn @ T(v)
+    if sums_from_outputs:
+        s4 = (G * O).sum(-1, keepdims=True)
+        s7d = (G * TO).sum(-1, keepdims=True) + (dOn * O).sum(-1, keepdims=True)
+    else:
+        s4 = (P * W).sum(-1, keepdims=True)
+        s7d = (P * (N * W + XY)).sum(-1, keepdims=True)
+    dTS = P * (W - s4)
+    dS = r(dTS * N + P * (XY - s7d))
+    dTS = r(dTS)
+    return {"dq": r(s * (dS @ k + dTS @ tk)), "dk": r(s * (T(dS) @ q + T(dTS) @ tq)),
+            "dtq": r(s * dTS @ k), "dtk": r(s * T(dTS) @ q)}
+
+
 def rel_frobenius(x, ref) -> float:
     """||x - ref||_F / ||ref||_F in fp64 (the accuracy gate's measure)."""
     x = _f64(x)
