@@ -30,7 +30,7 @@
  *     scale is an error.
  *   - The caller owns every buffer, including the workspace; the library allocates no device
  *     memory, keeps no pointer after returning, has no mutable global state (except the per-device
- *     address of sjvp_bwd_noalloc()'s static scratch), enqueues on the given hipStream_t (passed as
+ *     address of sjvp_bwd_noalloc()'s static scratch and the mode of sjvp_set_row_sum_repair()), enqueues on the given hipStream_t (passed as
  *     void*) of the CURRENT device and returns without synchronising.
  *   - Every function returns SJVP_OK (0) or a negative error code; nothing aborts or throws.
  *     Argument errors are detected before anything is launched.
@@ -103,7 +103,7 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
  * sjvp_bwd() picks its launches by shape: for Lk <= 128 and D <= 64 (rows 16-byte aligned) one
  * launch produces all six gradients and leaves the workspace untouched; otherwise the backward is
  * a row-owned launch (dq, dtq, and the row sums it leaves in the workspace) followed by a
- * column-owned one (dk, dv, dtk, dtv; two launches at D > 64), which consumes that workspace.
+ * column-owned one (dk, dv, dtk, dtv), which consumes that workspace.
  * sjvp_bwd_parts() runs the selected launches of that pair with sjvp_bwd()'s arguments;
  * sjvp_bwd_parts(SJVP_BWD_ALL, ...) is sjvp_bwd().  It has no counterpart in the reference: it exists
  * so that a profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only
@@ -163,6 +163,26 @@ int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq
                      const float* lse, const float* mu, void* dq, void* dk, void* dv, void* dtq,
                      void* dtk, void* dtv, int B, int H, int Lq, int Lk, int D,
                      const int64_t* strides /* [SJVP_B_COUNT*3] */, float scale, int dtype, void* stream);
+
+/*
+ * Row sums of the backward.  The reference forms sum_4 and sum_7 (the row sums of the cotangent on the
+ * tangent output) from the probabilities in a preprocess pass over the keys
+ * (flash_jvp_backward.py:2012-2290) and delta from the 16-bit output (flash_attn_triton.py:526-617).
+ * This library takes all of them from the 16-bit outputs o, to, which costs no pass, and the
+ * row-owned launch then measures what the rounding of o, to left in them (the sums over the keys of
+ * dS_dot and of dS, zero in exact arithmetic): it hands the column-owned launch the corrected sums,
+ * and repairs its own dq, dtq with one more pass over k (, tk) of the workgroups that need it.
+ *   SJVP_REPAIR_OFF     never run the second pass (dk, dtk still get the corrected sums)
+ *   SJVP_REPAIR_AUTO    (default) second pass where a row's residue exceeds the rounding of the tiles it
+ *                       is spread over: sharp attention rows, gradients formed by cancellation
+ *   SJVP_REPAIR_ALWAYS  second pass everywhere, and the row + column pair also for the shapes that
+ *                       would take the single launch, whose row sums stay those of the 16-bit outputs
+ *                       (not with sjvp_bwd_rotary): every gradient as accurate as the reference's form
+ * Process-wide; returns the previous mode, or SJVP_ERR_PARTS for an unknown one.  Calls already
+ * enqueued are not affected.
+ */
+enum sjvp_repair { SJVP_REPAIR_OFF = 0, SJVP_REPAIR_AUTO = 1, SJVP_REPAIR_ALWAYS = 2 };
+int sjvp_set_row_sum_repair(int mode);
 
 /* Bytes of caller-provided device scratch sjvp_bwd needs: lse in log2 units and the row sums sum_4
  * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,

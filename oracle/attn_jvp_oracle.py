@@ -331,7 +331,7 @@ def reference_rounding_error_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfl
 
 
 def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, sums_from_outputs=True,
-                           scale: Optional[float] = None) -> Dict[str, np.ndarray]:
+                           scale: Optional[float] = None, repaired: bool = False) -> Dict[str, np.ndarray]:
     """The query-side and key-side gradients with the two row sums of the backward formed either from
     the outputs rounded to ``dtype`` (``s4 = rowsum(G*O)``, ``s7d = rowsum(G*TO) + rowsum(dO*O)``: the
     FlashAttention "delta" form, extended to the cotangent on the tangent output) or from the
@@ -339,7 +339,14 @@ def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, s
     kernel does, flash_jvp_backward.py:2012-2290); everything else exact up to one rounding of the
     score-gradient tiles and of the results.  ``sum_j P (W - s4) = 0`` holds exactly only in the second
     form; in the first the rounding of O leaves a residue that is the same for every key of a row and
-    so adds up coherently in ``dS_dot^T Q`` and ``dS_dot K``.  Returns dq, dk, dtq, dtk."""
+    so adds up coherently in ``dS_dot^T Q`` and ``dS_dot K``.
+
+    ``repaired`` (with ``sums_from_outputs``) models what the row-owned + column-owned kernels do about
+    it: the residues ``rho4 = sum_j dS_dot``, ``rho7 = sum_j dS`` (zero with exact sums) are measured on
+    the unrounded tiles; the key side is formed with the corrected sums ``s4 + rho4``, ``s7d + rho7``; the
+    query side keeps the tiles formed with the rounded sums and subtracts ``s rho4 (P K)`` from dq_dot
+    and ``s (rho4 ((P*N) K + P K_dot) + rho7 (P K))`` from dq, with P and P*N rounded to ``dtype``.
+    Returns dq, dk, dtq, dtk."""
     r = lambda x: _round_to(x, dtype)
     q, k, v, tq, tk, tv, dOn, G = (r(_f64(x).numpy()) for x in (q, k, v, tq, tk, tv, dO, dTO))
     s = 1.0 / math.sqrt(q.shape[-1]) if scale is None else float(scale)
@@ -358,7 +365,18 @@ def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, s
         s4 = (P * W).sum(-1, keepdims=True)
         s7d = (P * (N * W + XY)).sum(-1, keepdims=True)
     dTS = P * (W - s4)
-    dS = r(dTS * N + P * (XY - s7d))
+    dS = dTS * N + P * (XY - s7d)
+    if repaired and sums_from_outputs:
+        rho4, rho7 = dTS.sum(-1, keepdims=True), dS.sum(-1, keepdims=True)
+        dTSc = P * (W - (s4 + rho4))
+        dSc = r(dTSc * N + P * (XY - (s7d + rho7)))
+        dTSc = r(dTSc)
+        dTSr, dSr, Pr, PNr = r(dTS), r(dS), r(P), r(P * N)
+        PK = Pr @ k
+        return {"dq": r(s * (dSr @ k + dTSr @ tk - rho4 * (PNr @ k + Pr @ tk) - rho7 * PK)),
+                "dk": r(s * (T(dSc) @ q + T(dTSc) @ tq)),
+                "dtq": r(s * (dTSr @ k - rho4 * PK)), "dtk": r(s * T(dTSc) @ q)}
+    dS = r(dS)
     dTS = r(dTS)
     return {"dq": r(s * (dS @ k + dTS @ tk)), "dk": r(s * (T(dS) @ q + T(dTS) @ tq)),
             "dtq": r(s * dTS @ k), "dtk": r(s * T(dTS) @ q)}

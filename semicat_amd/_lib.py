@@ -34,8 +34,12 @@ F_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to")
 B_TENSORS = ("q", "k", "v", "tq", "tk", "tv", "o", "to", "dO", "dTO",
              "dq", "dk", "dv", "dtq", "dtk", "dtv")
 
+SJVP_REPAIR_OFF = 0
+SJVP_REPAIR_AUTO = 1
+SJVP_REPAIR_ALWAYS = 2
+
 EXPORTS = ("sjvp_fwd", "sjvp_bwd", "sjvp_bwd_parts", "sjvp_bwd_noalloc", "sjvp_fwd_rotary", "sjvp_bwd_rotary", "sjvp_bwd_workspace_bytes", "sjvp_rope",
-           "sjvp_strerror", "sjvp_version", "sjvp_build_id")
+           "sjvp_set_row_sum_repair", "sjvp_strerror", "sjvp_version", "sjvp_build_id")
 
 _lock = threading.Lock()
 _lib = None
@@ -82,6 +86,8 @@ def load() -> ctypes.CDLL:
             vpp = ctypes.POINTER(ctypes.c_void_p)
             lib.sjvp_rope.argtypes = [i, vpp, vpp, i64p, vp, vp, ctypes.c_int64] + [i] * 8 + [vp]
             lib.sjvp_rope.restype = i
+            lib.sjvp_set_row_sum_repair.argtypes = [i]
+            lib.sjvp_set_row_sum_repair.restype = i
             lib.sjvp_strerror.argtypes = [i]
             lib.sjvp_strerror.restype = ctypes.c_char_p
             lib.sjvp_version.argtypes = []

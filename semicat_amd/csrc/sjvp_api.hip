@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <math.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "sjvp_launch.hpp"
@@ -67,11 +68,17 @@ int check_rotary(const float* cos, const float* sin, int64_t cs_stride, int tabl
 
 inline float resolve_scale(float scale, int D) { return scale > 0.f ? scale : 1.0f / sqrtf((float)D); }
 
+// Process-wide setting of sjvp_set_row_sum_repair().
+std::atomic<int> g_row_sum_repair{SJVP_REPAIR_AUTO};
+
 // Kernel selection of the backward: the single launch where it fits, else the row + column pair.
 template <typename T>
 int bwd_select(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, hipStream_t stream) {
     if (!p.vec) return bwd_pair_any<T>(p, BH, has_do, has_g, parts, stream);
-    if (parts == SJVP_BWD_ALL && p.Lk <= kOwned16 && p.D <= 64) return bwd_fused<T>(p, BH, has_do, has_g, stream);
+    // the single launch takes its row sums from the 16-bit outputs and cannot repair them: a caller who
+    // asked for the repair everywhere gets the pair (the folded rotation exists in the single launch only)
+    const bool single = parts == SJVP_BWD_ALL && p.Lk <= kOwned16 && p.D <= 64;
+    if (single && (p.rowfix != SJVP_REPAIR_ALWAYS || p.rope.cos)) return bwd_fused<T>(p, BH, has_do, has_g, stream);
     return bwd_pair_vec<T>(p, BH, has_do, has_g, parts, stream);
 }
 
@@ -173,6 +180,8 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
     p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
     p.rope = rope;
+    p.rowfix = g_row_sum_repair.load(std::memory_order_relaxed);
+    p.rowfix_tau = dtype == SJVP_FP16 ? 0x1p-11f : 0x1p-8f;  // unit roundoff of the tiles' 16-bit format
     if (rope.cos && (!p.vec || parts != SJVP_BWD_ALL)) return SJVP_ERR_ROTARY;  // the single launch only
 
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -435,6 +444,11 @@ int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* stride
     return by_out(Fp16{});
 }
 
+int sjvp_set_row_sum_repair(int mode) {
+    if (mode < SJVP_REPAIR_OFF || mode > SJVP_REPAIR_ALWAYS) return SJVP_ERR_PARTS;
+    return g_row_sum_repair.exchange(mode);
+}
+
 const char* sjvp_strerror(int status) {
     switch (status) {
         case SJVP_OK: return "ok";
@@ -445,7 +459,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than sjvp_bwd_workspace_bytes()";
         case SJVP_ERR_LAUNCH: return "HIP kernel launch failed";
         case SJVP_ERR_COTANGENT: return "at least one of dO and dTO must be given";
-        case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL";
+        case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL (sjvp_set_row_sum_repair: mode must be SJVP_REPAIR_OFF, _AUTO or _ALWAYS)";
         case SJVP_ERR_SCALE: return "scale must be finite and >= 0 (0 selects 1/sqrt(D))";
         case SJVP_ERR_SCRATCH: return "sjvp_bwd_noalloc: B * H * ceil(Lq/128)*128 exceeds SJVP_NOALLOC_MAX_ROWS, or the static scratch could not be located on this device";
         case SJVP_ERR_ROTARY: return "rotary embedding: sjvp_rope needs n in 1..4, rot_dim even with 2 <= rot_dim <= D, and no mix of bf16 and fp16; sjvp_fwd_rotary / sjvp_bwd_rotary need D = 64, Lk <= 128, bf16 or fp16 tensors with 16-byte aligned rows, and 16-byte aligned fp32 tables of at least max(Lq, Lk) rows with a row stride that is a multiple of 4";

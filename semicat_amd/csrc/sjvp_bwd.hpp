@@ -40,6 +40,8 @@ struct BwdParams {
     float scale;
     int vec;
     RopeTables rope;  // q, k (and tangents) are rotated as they are loaded, their gradients rotated back
+    int rowfix;        // repair of dQ, dQ_dot for the residues of the row sums: 0 never, 1 where needed, 2 always
+    float rowfix_tau;  // a residue counts once it exceeds this fraction of the row's absolute tile sum
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -224,9 +226,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         p.s7d[so] = s7d;
     }
     for (int i = 0; i < n; ++i) {
-        __syncthreads();  // the previous stage is fully consumed
+        workgroup_barrier();  // the previous stage is fully consumed
         fill(i);
-        __syncthreads();
+        workgroup_barrier();
         if (!wave_active) continue;
         const int k0 = i * kStageRows;
         if (k0 + kStageRows > p.Lk) compute(k0, std::true_type{});
@@ -434,9 +436,9 @@ __global__ __launch_bounds__(kThreads, (DO_K && DO_V && HAS_G) ? 1 : 2) void bwd
 
     const int n = (p.Lq + kStageRows - 1) / kStageRows;
     for (int i = 0; i < n; ++i) {
-        __syncthreads();  // the previous stage is fully consumed
+        workgroup_barrier();  // the previous stage is fully consumed
         fill(i);
-        __syncthreads();
+        workgroup_barrier();
         if (wave_active) compute();
     }
     {

@@ -371,7 +371,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // Only the own rows and stage 0 are waited for here; the later stages are issued once these
     // have landed, so that their copies run under the arithmetic instead of ahead of it.
     wait_stages<SPT>(0);
-    __syncthreads();
+    workgroup_barrier();
     if (issued < ns) issue_next();
     // ROPE: Q (, Q_dot) of a landed stage, one item per thread of the upper half of the workgroup
     auto rotate_stage = [&](elem_t* slot, int row0) {
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             const int slab = it >> 7;
             rope_slab_item<T>(ownK + slab * SE, it & 127, p.rope, 32 * (slab & 3), 1.0f);
         }
-        __syncthreads();
+        workgroup_barrier();
     }
     {
         const int r = 16 * (wave & 1) + n;
@@ -406,13 +406,13 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     for (int i = 0; i < ns; ++i) {
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
-        __syncthreads();
+        workgroup_barrier();
         if (i >= 1) flush_rows((i - 1) * kStageRows);
         if (issued < ns && issued < i + R) issue_next();  // into the slot of stage issued - R <= i - 1
         elem_t* slot = ring + (i % R) * SM::slot;
         if (wave_active) tile(slot);
         if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
-        __syncthreads();
+        workgroup_barrier();
         if (i + 1 < ns) {
             row_sums(ring + ((i + 1) % R) * SM::slot);
             rotate_stage(ring + ((i + 1) % R) * SM::slot, (i + 1) * kStageRows);
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
         else row_outputs(i * kStageRows, std::false_type{});
     }
-    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     flush_rows((ns - 1) * kStageRows);
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;

@@ -8,6 +8,20 @@
 // The owned rows are loaded straight into registers (each lane its own 16-byte pieces), the streamed
 // side goes through an LDS ring filled by LDS-DMA.  Each gradient is accumulated in fp32 registers by
 // exactly one wavefront and written once: deterministic, no atomics.
+//
+// Row sums.  The row-owned kernel starts from s4' = rowsum(G*O), s7d' = rowsum(G*TO) + rowsum(dO*O),
+// formed from the 16-bit outputs, whose rounding leaves s4' = s4 + e4, s7d' = s7d + e7.  With the exact
+// sums, sum_j dS_dot_ij = sum_j dS_ij = 0 for every query i; with the rounded ones the sums over the
+// keys come out as rho4 = -e4 and rho7 = -e7.  A wave owns whole query rows, so it accumulates both
+// residues in fp32 beside its tiles (per-lane adds) and
+//   - leaves the corrected sums s4' + rho4, s7d' + rho7 in the workspace: the column-owned kernel
+//     works with sums as accurate as the ones the reference's preprocess kernel forms from the
+//     probabilities (semicat/jvp_utils/flash_jvp_backward.py:2266-2287);
+//   - repairs its own dQ_dot, dQ, which were accumulated with the rounded sums and therefore carry
+//     -s rho4 (P K) and -s (rho4 ((P*N) K + P K_dot) + rho7 (P K)): where a residue is not small against
+//     the row's |dS_dot| / |dS| mass (sharp rows, gradients formed by cancellation), the workgroup
+//     streams K (, K_dot) a second time, forms P K and (P*N) K + P K_dot, and subtracts
+//     (BwdParams::rowfix: 0 never, 1 where the residues call for it, 2 always).
 #pragma once
 #include "sjvp_bwd.hpp"
 #include "sjvp_w16.hpp"
@@ -117,13 +131,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
     const float lse2 = p.lse[so] * kLog2e;
     const float mu = HAS_G ? p.mu[so] : 0.f;
-    if (g == 0) {
-        // every row below Lr is written (zeros beyond Lq except lse2, which is finite): the
-        // column-owned kernel, which runs after this one, stages 32-row groups
-        p.lse2[so] = lse2;
-        p.s4[so] = s4;
-        p.s7d[so] = s7d;
-    }
+    // every row below Lr gets its workspace entries (zeros beyond Lq except lse2, which is finite): the
+    // column-owned kernel, which runs after this one, stages 32-row groups
+    if (g == 0) p.lse2[so] = lse2;
     const float sl2 = p.scale * kLog2e;
     f32x4 dq[DT], dtq[DT];
 #pragma unroll
@@ -131,6 +141,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         dq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         dtq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    // this lane's part of sum_j dS_dot_ij, sum_j dS_ij (zero in exact arithmetic), and of their absolute
+    // sums, which only set the scale of a threshold and are sampled on every fourth key
+    float r4 = 0.f, r7 = 0.f, a4 = 0.f, a7 = 0.f;
 
     auto compute = [&](const elem_t* slot, int k0) {
         const elem_t* sK = slot;
@@ -174,9 +187,13 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                     const float dts = pj * (w[t][j] - s4);
                     w[t][j] = dts;
                     xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s7d));
+                    r4 += dts;
+                    if (j == 0) a4 += fabsf(dts);
                 } else {
                     xy[t][j] = pj * (xy[t][j] - s7d);
                 }
+                r7 += xy[t][j];
+                if (j == 0) a7 += fabsf(xy[t][j]);
             }
         };
         // the second key tile's MFMA chains run under the first tile's element-wise arithmetic
@@ -217,11 +234,110 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         // copies issued after stage i: the later stages; anything else in flight (the own rows'
         // loads, the statistics) only makes the wait stricter
         wait_stages<SPT>(issued - 1 - i);
-        __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+        workgroup_barrier();  // stage i has landed for every wave; stage i-1 is fully consumed
         if (i > 0 && issued < ns) issue_next();
         if (wave_active) compute(ring + (i % R) * SM::slot, i * kStageRows);
     }
-    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    // the residues of the row sums (see the top of the file); the four lanes of a query hold its keys
+    r4 = group_sum(r4);
+    r7 = group_sum(r7);
+    a4 = 4.0f * group_sum(a4);
+    a7 = 4.0f * group_sum(a7);
+    if (g == 0) {
+        p.s4[so] = s4 + r4;
+        p.s7d[so] = s7d + r7;
+    }
+    // A residue matters where it is not small against the rounding of the tiles it is spread over:
+    // |rho| against tau * sum_j |tile_ij|, tau = the spacing of the 16-bit format.  NaN compares false.
+    const bool wanted = qvalid && (fabsf(r4) > p.rowfix_tau * a4 || fabsf(r7) > p.rowfix_tau * a7);
+    const bool repair = p.rowfix == 2 || (p.rowfix == 1 && workgroup_barrier_or(wanted));
+    if (repair) {
+        // Second pass over the keys: P K into pk and (P*N) K + P K_dot into t2, with the 16-bit P and P*N
+        // as B operands (the terms they correct are themselves small).
+        workgroup_barrier();  // every wave is done with the ring of the first pass
+        using Plan2 = CopyPlan<HD, HAS_G ? 2 : 1, 1, kXThreads16>;
+        constexpr int SPT2 = Plan2::N;
+        Plan2 plan2;
+        if constexpr (HAS_G)
+            plan2.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl}, Src{p.tk.head(b, h), p.tk.sl});
+        else
+            plan2.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl});
+        int issued2 = 0;
+        auto issue2 = [&]() {
+            plan2.issue(ring + (issued2 % R) * SM::slot, p.Lk - issued2 * kStageRows);
+            ++issued2;
+        };
+        while (issued2 < R && issued2 < ns) issue2();
+        f32x4 pk[DT], t2[DT];
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            pk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            t2[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        auto compute2 = [&](const elem_t* slot, int k0) {
+            const elem_t* sK = slot;
+            const elem_t* sTK = slot + SE;
+            f32x4 s[2], ts[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+                ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < KC; ++c) {
+                    const u32x4 ak = lds_a_rows16<HD>(sK, t, c, n, g);
+                    s[t] = T::mfma16(ak, qB[c], s[t]);
+                    if constexpr (HAS_G) {
+                        ts[t] = T::mfma16(ak, tqB[c], ts[t]);
+                        const u32x4 atk = lds_a_rows16<HD>(sTK, t, c, n, g);
+                        ts[t] = T::mfma16(atk, qB[c], ts[t]);
+                    }
+                }
+            }
+            const bool ragged = k0 + kStageRows > p.Lk;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float pj = fast_exp2(fmaf(s[t][j], sl2, -lse2));
+                    if (ragged && k0 + 16 * t + 4 * g + j >= p.Lk) pj = 0.f;
+                    s[t][j] = pj;
+                    if constexpr (HAS_G) ts[t][j] = pj * fmaf(ts[t][j], p.scale, -mu);
+                }
+            }
+            const u32x4 pB = pack_b16<T>(s[0], s[1]);
+            u32x4 pnB;
+            if constexpr (HAS_G) pnB = pack_b16<T>(ts[0], ts[1]);
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                const u32x4 ak = lds_a_tr16<HD>(sK, 16 * d, lane);
+                pk[d] = T::mfma16(ak, pB, pk[d]);
+                if constexpr (HAS_G) {
+                    t2[d] = T::mfma16(ak, pnB, t2[d]);
+                    const u32x4 atk = lds_a_tr16<HD>(sTK, 16 * d, lane);
+                    t2[d] = T::mfma16(atk, pB, t2[d]);
+                }
+            }
+        };
+        for (int i = 0; i < ns; ++i) {
+            wait_stages<SPT2>(issued2 - 1 - i);
+            workgroup_barrier();
+            if (i > 0 && issued2 < ns) issue2();
+            if (wave_active) compute2(ring + (i % R) * SM::slot, i * kStageRows);
+        }
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (HAS_G) {
+                    dtq[d][j] = fmaf(-r4, pk[d][j], dtq[d][j]);
+                    dq[d][j] -= fmaf(r4, t2[d][j], r7 * pk[d][j]);
+                } else {
+                    dq[d][j] = fmaf(-r7, pk[d][j], dq[d][j]);
+                }
+            }
+        }
+    }
+    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = q0 + wave * 16;
@@ -459,11 +575,11 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
 
     for (int i = 0; i < ns; ++i) {
         wait_stages<SPT>(issued - 1 - i);
-        __syncthreads();  // stage i has landed for every wave; stage i-1 is fully consumed
+        workgroup_barrier();  // stage i has landed for every wave; stage i-1 is fully consumed
         if (i > 0 && issued < ns) issue_next();
         if (wave_active) compute(ring + (i % R) * SM::slot);
     }
-    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     if (!wave_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
     const int row0 = key0 + wave * 16;
@@ -674,14 +790,14 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
 
     for (int i = 0; i < ns; ++i) {
         wait_stages<SPT>(issued - 1 - i);
-        __syncthreads();  // stage i has landed for every wave; stage i-1 and the exchange area are free
+        workgroup_barrier();  // stage i has landed for every wave; stage i-1 and the exchange area are free
         if (i > 0 && issued < ns) issue_next();
         const elem_t* slot = ring + (i % R) * SM::slot;
         if (pair_active) scores(slot);
-        __syncthreads();  // the partner's tiles are visible
+        workgroup_barrier();  // the partner's tiles are visible
         if (pair_active) outputs(slot);
     }
-    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     if (!pair_active) return;
     elem_t* stage_tile = ring + wave * StoreStage16<64>::elems;
     const int row0 = key0 + pr * 16;

@@ -119,6 +119,21 @@ struct RopeTables {
     int rows;          // rows of the tables (positions beyond are clamped; their data is zero padding)
 };
 
+// Workgroup barrier.  __syncthreads() leaves the wait for this wave's own LDS writes to the compiler,
+// and at the head of a loop the compiler has been seen to hoist that wait into the loop's preheader
+// only, so that a wave reached the barrier with the LDS write that ends its loop body still queued
+// and another wave read the old value behind the barrier (one 16 x 16 tile of dQ in one of some ten
+// thousand).  The explicit s_waitcnt lgkmcnt(0) is kept by the compiler wherever the barrier goes.
+__device__ __forceinline__ void workgroup_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0); vmcnt and expcnt untouched
+    __syncthreads();
+}
+// The same with a vote: true if `pred` holds for any thread of the workgroup.
+__device__ __forceinline__ bool workgroup_barrier_or(bool pred) {
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    return __syncthreads_or(pred) != 0;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

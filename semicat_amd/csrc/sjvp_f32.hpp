@@ -149,14 +149,14 @@ __global__ __launch_bounds__(kF32Threads) void fwd_f32_kernel(const FwdParamsF32
     float m_i = -INFINITY, l_i = 0.f, mu_i = 0.f;  // running maximum (log2 units), exp-sum, sum p * S_dot
 
     for (int k0 = 0; k0 < p.Lk; k0 += kF32Tile) {
-        __syncthreads();
+        workgroup_barrier();
         f32_fill_tile<HD>(sK, p.k.head(b, h), p.k.sl, k0, p.Lk, p.D, tid);
         f32_fill_tile<HD>(sV, p.v.head(b, h), p.v.sl, k0, p.Lk, p.D, tid);
         if constexpr (JVP) {
             f32_fill_tile<HD>(sTK, p.tk.head(b, h), p.tk.sl, k0, p.Lk, p.D, tid);
             f32_fill_tile<HD>(sTV, p.tv.head(b, h), p.tv.sl, k0, p.Lk, p.D, tid);
         }
-        __syncthreads();
+        workgroup_barrier();
         float s[kF32Tile], ts[kF32Tile];
         float mloc = -INFINITY;
 #pragma unroll
@@ -261,14 +261,14 @@ __global__ __launch_bounds__(kF32Threads) void bwd_row_f32_kernel(const BwdParam
     }
     const float sl2 = p.scale * kLog2e;
     for (int k0 = 0; k0 < p.Lk; k0 += kF32Tile) {
-        __syncthreads();
+        workgroup_barrier();
         f32_fill_tile<HD>(sK, p.k.head(b, h), p.k.sl, k0, p.Lk, p.D, tid);
         f32_fill_tile<HD>(sV, p.v.head(b, h), p.v.sl, k0, p.Lk, p.D, tid);
         if constexpr (HAS_G) {
             f32_fill_tile<HD>(sTK, p.tk.head(b, h), p.tk.sl, k0, p.Lk, p.D, tid);
             f32_fill_tile<HD>(sTV, p.tv.head(b, h), p.tv.sl, k0, p.Lk, p.D, tid);
         }
-        __syncthreads();
+        workgroup_barrier();
 #pragma unroll 4
         for (int j = 0; j < kF32Tile; ++j) {
             const float s = sum8(f32_dot<HD>(q, sK, j, c));
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(kF32Threads) void bwd_col_f32_kernel(const BwdParam
     }
     const float sl2 = p.scale * kLog2e;
     for (int q0 = 0; q0 < p.Lq; q0 += kF32Tile) {
-        __syncthreads();
+        workgroup_barrier();
         f32_fill_tile<HD>(sQ, p.q.head(b, h), p.q.sl, q0, p.Lq, p.D, tid);
         if constexpr (HAS_G) {
             f32_fill_tile<HD>(sTQ, p.tq.head(b, h), p.tq.sl, q0, p.Lq, p.D, tid);
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(kF32Threads) void bwd_col_f32_kernel(const BwdParam
             // rows below Lr exist in every statistic; mu is absent without a cotangent on TO
             sStat[tid] = (which == 1 && !HAS_G) ? 0.f : src[(int64_t)bh * p.Lr + q0 + r];
         }
-        __syncthreads();
+        workgroup_barrier();
 #pragma unroll 4
         for (int i = 0; i < kF32Tile; ++i) {
             const float s = sum8(f32_dot<HD>(k, sQ, i, c));

@@ -201,9 +201,9 @@ __global__ __launch_bounds__(kThreads, 1) void fwd_kernel(const FwdParams p) {
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
     for (int i = 0; i < n; ++i) {
-        __syncthreads();  // the previous stage is fully consumed
+        workgroup_barrier();  // the previous stage is fully consumed
         fill(i);
-        __syncthreads();
+        workgroup_barrier();
         if (!wave_active) continue;
         const int k0 = i * kStageRows;
         if (k0 + kStageRows > p.Lk) compute(k0, std::true_type{});

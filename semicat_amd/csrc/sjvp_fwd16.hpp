@@ -104,7 +104,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
 
     // SPB = 1: the own rows and stage 0 were issued before the other stages; SPB = 2: everything
     wait_stages<SPT>(SPB == 2 ? 0 : issued - 1);
-    __syncthreads();
+    workgroup_barrier();
     u32x4 qB[KC], tqB[KC];
     {
         const int r = 16 * (wave & 1) + n;
@@ -121,14 +121,14 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
         if constexpr (ROPE) {
             if (tid < 128) rope_slab_item<T>(slot, tid, p.rope, k0, 1.0f);
             else if (JVP && tid < 256) rope_slab_item<T>(slot + 2 * SE, tid - 128, p.rope, k0, 1.0f);
-            __syncthreads();
+            workgroup_barrier();
         }
     };
     rotate_stage(ring, 0);
     if constexpr (SPB == 2) {
         // the operands must have arrived in registers before the copies below overwrite their slots
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __syncthreads();
+        workgroup_barrier();
         while (issued < R && issued < ns) issue_next();
     }
 
@@ -216,7 +216,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
             if (i > 0) {
                 // the stages of this step have landed for every wave; those of the last step are consumed
                 wait_stages<SPT>(SPB == 2 ? 0 : issued - 1 - i);
-                __syncthreads();
+                workgroup_barrier();
 #pragma unroll
                 for (int u = 0; u < SPB; ++u)
                     if (issued < ns) issue_next();
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
                 if (i + u < ns) compute(ring + (h + u) * SM::slot, (i + u) * kStageRows);
         }
     }
-    __syncthreads();  // every wave is done reading the ring: it becomes the store staging area
+    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     const int64_t so = (int64_t)bh * p.Lr + qrow;
     if (!wave_active) {
         // All 16 rows of this wave lie beyond Lq: their statistic rows get the values a zero query

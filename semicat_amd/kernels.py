@@ -66,6 +66,21 @@ def rotary_fusable(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, others: 
     return True
 
 
+_REPAIR_MODES = {"off": _lib.SJVP_REPAIR_OFF, "auto": _lib.SJVP_REPAIR_AUTO, "always": _lib.SJVP_REPAIR_ALWAYS}
+
+
+def set_row_sum_repair(mode: str) -> str:
+    """How the backward deals with what the rounding of ``o``, ``to`` leaves in its row sums (the
+    reference forms those sums from the probabilities, flash_jvp_backward.py:2012-2290): ``"off"``,
+    ``"auto"`` (default: a second pass over the keys for the workgroups whose rows need it) or
+    ``"always"`` (everywhere, and the row + column launches also where the single launch would run).
+    Process-wide; returns the previous mode."""
+    if mode not in _REPAIR_MODES:
+        raise ValueError(f"row-sum repair mode must be one of {sorted(_REPAIR_MODES)}, got {mode!r}")
+    prev = _lib.load().sjvp_set_row_sum_repair(_REPAIR_MODES[mode])
+    return {v: k for k, v in _REPAIR_MODES.items()}[prev]
+
+
 def stat_rows(L: int) -> int:
     """Length of the row-statistic buffers: L rounded up to 128 (ryu_triton.py:351)."""
     return ((L + 127) // 128) * 128

@@ -221,3 +221,31 @@ def test_row_sums_from_rounded_outputs_leave_a_coherent_residue():
     for form in (False, True):
         m = orc.row_sum_rounding_model(*[x[n] for n in orc.TENSOR_ORDER], sums_from_outputs=form)
         assert max(orc.rel_frobenius(torch.from_numpy(v), ref[n]) for n, v in m.items()) <= 6e-3
+
+
+def test_repaired_row_sums_match_the_sums_from_the_probabilities():
+    """The repaired form of the row-sum model (residues of dS_dot, dS summed over the keys, corrected
+    sums for the key side, P K and (P*N) K + P K_dot terms for the query side) is as accurate as the
+    reference's form on the cases where the sums of the rounded outputs alone fail: the 255-key case,
+    a saturated single row in fp16 (0.9998 of the probability on one of five keys: 0.5-0.6 relative
+    error without the repair) and constructed saturated rows in bf16."""
+    cases = []
+    x = orc.make_inputs(2, 1, 2, 255, 40, seed=1062, primal_scale=2.0, tangent_scale=0.3, dtype=torch.bfloat16)
+    cases.append((x, torch.bfloat16, 1e-2))
+    x = orc.make_inputs(1, 1, 1, 5, 80, seed=1029, primal_scale=2.0, tangent_scale=0.3, dtype=torch.float16)
+    cases.append((x, torch.float16, 0.3))
+    x = orc.make_inputs(1, 2, 3, 133, 80, seed=5, primal_scale=1.0, tangent_scale=0.3, dtype=torch.bfloat16)
+    for i in range(3):
+        x["k"][:, :, 7 + 40 * i, :] = (x["q"][:, :, i, :].float() * 1.5).to(torch.bfloat16)
+    cases.append((x, torch.bfloat16, 0.3))
+    for x, dtype, unrepaired_floor in cases:
+        args = [x[n] for n in orc.TENSOR_ORDER]
+        ref = orc.attention_jvp_autograd(*args)
+        err = {}
+        for label, kw in (("exact", dict(sums_from_outputs=False)), ("delta", dict()), ("repaired", dict(repaired=True))):
+            m = orc.row_sum_rounding_model(*args, dtype=dtype, **kw)
+            err[label] = {n: orc.rel_frobenius(torch.from_numpy(v), ref[n]) for n, v in m.items()}
+        assert max(err["delta"].values()) >= unrepaired_floor, err
+        for n in ("dq", "dk", "dtq", "dtk"):
+            assert err["repaired"][n] <= 2.0 * err["exact"][n] + 2e-4, (n, err)
+            assert err["repaired"][n] <= 5e-3, (n, err)
