@@ -183,7 +183,6 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--graph", action="store_true",
                     help="replay a HIP graph of one step instead of launching through the C ABI every step")
-    ap.add_argument("--no-graph", action="store_true", help="(default behaviour; kept for old command lines)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache timing over rotating buffer sets")
     ap.add_argument("--no-hardware", action="store_true", help="skip the copy / GEMM measurement of the box")
@@ -268,8 +267,11 @@ def main() -> int:
             bwd()
             e[2].record(stream)
         stream.synchronize()
-        fwd_raw_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / n_ev
-        bwd_raw_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / n_ev
+        fwd_each = sorted(e[0].elapsed_time(e[1]) for e in evs)
+        bwd_each = sorted(e[1].elapsed_time(e[2]) for e in evs)
+        step_each = sorted(e[0].elapsed_time(e[2]) for e in evs)
+        fwd_raw_ms = sum(fwd_each) / n_ev
+        bwd_raw_ms = sum(bwd_each) / n_ev
         # An event between two kernels keeps them a few microseconds apart, which the plain steps of
         # the timed region do not pay: the instrumented step is that much longer than the timed one.
         # Each kernel's interval holds one such gap; it is taken out in equal parts so that the two
@@ -378,7 +380,14 @@ def main() -> int:
         "autograd_step_ms": autograd_ms,
         "fwd_ms": fwd_ms,
         "bwd_ms": bwd_ms,
-        "event_intervals_ms": {"fwd": fwd_raw_ms, "bwd": bwd_raw_ms, "gap_removed_per_kernel": gap_ms},
+        "event_intervals_ms": {"fwd": fwd_raw_ms, "bwd": bwd_raw_ms, "gap_removed_per_kernel": gap_ms,
+                               # median and minimum over the instrumented steps (event gaps included)
+                               "fwd_median": fwd_each[n_ev // 2], "fwd_min": fwd_each[0],
+                               "bwd_median": bwd_each[n_ev // 2], "bwd_min": bwd_each[0],
+                               "step_median": step_each[n_ev // 2], "step_min": step_each[0]},
+        # the forward by the count of the reference's own harness (10*B*H*L^2*D, ryu_triton.py:1000-1003,
+        # which under-counts its six contractions), for comparison with figures quoted that way
+        "fwd_TFLOPs_by_reference_count": 10.0 * BH * L * L * D / (fwd_ms * 1e-3) / 1e12,
         "cold_ms_per_step": cold_ms,
         "cold_tflops": None if cold_ms is None else step_flops() / (cold_ms * 1e-3) / 1e12,
         "kernels": {n: {"ms": w["ms"], "GBps": w["GBps"], "TFLOPs": w["TFLOPs"]} for n, w in work.items()},

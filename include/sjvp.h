@@ -60,7 +60,7 @@ enum sjvp_status {
     SJVP_ERR_LAUNCH = -6,    /* the HIP runtime refused a launch (status of hipLaunchKernel) */
     SJVP_ERR_COTANGENT = -7, /* sjvp_bwd called with both dO and dTO NULL                    */
     SJVP_ERR_PARTS = -8,     /* sjvp_bwd_parts: parts is not a combination of sjvp_bwd_part  */
-    SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 2 or > D, or dtypes that mix bf16 and fp16;
+    SJVP_ERR_ROTARY = -9,    /* sjvp_rope: n outside 1..4, rot_dim odd, < 0 or > D, or dtypes that mix bf16 and fp16;
                                 sjvp_fwd_rotary / sjvp_bwd_rotary: a shape, dtype or table they do not serve */
     SJVP_ERR_SCALE = -10,    /* scale negative, infinite or NaN (0 selects the default)      */
     SJVP_ERR_SCRATCH = -11   /* sjvp_bwd_noalloc: problem beyond SJVP_NOALLOC_MAX_ROWS, or no static scratch on this device */
@@ -202,7 +202,9 @@ size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
  *   x[i], y[i]   [B,H,L,D] views, unit last stride; strides[6*i + {0,1,2}] = (batch, head, sequence)
  *                element strides of x[i], strides[6*i + {3,4,5}] those of y[i]; y[i] may alias x[i]
  *                only if both have the same dtype and strides
- *   cos, sin     fp32 [L][rot_dim/2] with row stride cs_stride (elements)
+ *   cos, sin     fp32 [L][rot_dim/2] with row stride cs_stride (elements); rot_dim = 0 makes the call a
+ *                plain cast / layout change of up to four tensors in one launch (cos, sin may be NULL):
+ *                the casts that functional.py:318-322,330-331 put around the op for float32 callers
  *   in_dtype, out_dtype   SJVP_BF16, SJVP_FP16 or SJVP_FP32 (not bf16 on one side and fp16 on the other)
  */
 int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides /* [n*6] */,

@@ -49,7 +49,11 @@ int check_common(int B, int H, int Lq, int Lk, int D, int dtype, float scale) {
     if (dtype < SJVP_BF16 || dtype > SJVP_FP32_BF16) return SJVP_ERR_DTYPE;
     if (B < 1 || H < 1 || Lq < 1 || Lk < 1) return SJVP_ERR_SHAPE;
     if (D < 16 || D > 128) return SJVP_ERR_HEAD_DIM;
-    const int64_t blocks = (int64_t)B * H * ((int64_t)round_up(Lq > Lk ? Lq : Lk, 32) / 32);
+    // the finest launch takes one workgroup per 32 rows of the longer axis rounded up to 128 (the
+    // statistic rows): that grid, in 64 bits, has to fit the 31 bits of a launch dimension
+    const int64_t longer = Lq > Lk ? Lq : Lk;
+    if (longer > (1LL << 30)) return SJVP_ERR_SHAPE;  // keeps the 32-bit round-ups below exact
+    const int64_t blocks = (int64_t)B * H * ((longer + 127) / 128 * 4);
     if (blocks > 0x7fffffffLL) return SJVP_ERR_SHAPE;
     if (!(scale >= 0.f) || isinf(scale)) return SJVP_ERR_SCALE;  // 0 selects the default; NaN fails too
     return SJVP_OK;
@@ -68,8 +72,23 @@ int check_rotary(const float* cos, const float* sin, int64_t cs_stride, int tabl
 
 inline float resolve_scale(float scale, int D) { return scale > 0.f ? scale : 1.0f / sqrtf((float)D); }
 
+constexpr int kMaxDevices = 64;
+
 // Process-wide setting of sjvp_set_row_sum_repair().
 std::atomic<int> g_row_sum_repair{SJVP_REPAIR_AUTO};
+
+// Compute units of the current device (looked up once per device).
+int compute_units() {
+    static std::atomic<int> cached[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 // Kernel selection of the backward: the single launch where it fits, else the row + column pair.
 template <typename T>
@@ -78,7 +97,12 @@ int bwd_select(const BwdParams& p, int BH, bool has_do, bool has_g, int parts, h
     // the single launch takes its row sums from the 16-bit outputs and cannot repair them: a caller who
     // asked for the repair everywhere gets the pair (the folded rotation exists in the single launch only)
     const bool single = parts == SJVP_BWD_ALL && p.Lk <= kOwned16 && p.D <= 64;
-    if (single && (p.rowfix != SJVP_REPAIR_ALWAYS || p.rope.cos)) return bwd_fused<T>(p, BH, has_do, has_g, stream);
+    // The single launch is one workgroup per (batch, head) pair walking the whole query axis: a few
+    // pairs with a long query axis would leave most of the chip idle, while the row-owned launch of the
+    // pair spreads the queries over Lq / 64 workgroups per pair.
+    const bool few_long = 2 * BH <= compute_units() && p.Lq >= 4 * kOwned16 && !p.rope.cos;
+    if (single && !few_long && (p.rowfix != SJVP_REPAIR_ALWAYS || p.rope.cos))
+        return bwd_fused<T>(p, BH, has_do, has_g, stream);
     return bwd_pair_vec<T>(p, BH, has_do, has_g, parts, stream);
 }
 
@@ -197,7 +221,6 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
 // looked up once per device, with that device current.
 static __device__ __align__(256) __attribute__((used)) float scratch[3 * (size_t)SJVP_NOALLOC_MAX_ROWS];
 
-constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 float* g_scratch_ptr[kMaxDevices] = {};
 
@@ -385,10 +408,11 @@ int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq
 int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* strides, const float* cos,
               const float* sin, int64_t cs_stride, int B, int H, int L, int D, int rot_dim, int in_dtype,
               int out_dtype, int inverse, void* stream) {
-    if (!x || !y || !strides || !cos || !sin) return SJVP_ERR_NULL;
+    if (!x || !y || !strides) return SJVP_ERR_NULL;
+    if (rot_dim != 0 && (!cos || !sin)) return SJVP_ERR_NULL;  // rot_dim 0: cast / layout change only
     if (n < 1 || n > kRopeMaxTensors) return SJVP_ERR_ROTARY;
     if (B < 1 || H < 1 || L < 1 || D < 1) return SJVP_ERR_SHAPE;
-    if (rot_dim < 2 || rot_dim > D || (rot_dim & 1)) return SJVP_ERR_ROTARY;
+    if (rot_dim < 0 || rot_dim > D || (rot_dim & 1)) return SJVP_ERR_ROTARY;
     auto known = [](int d) { return d == SJVP_BF16 || d == SJVP_FP16 || d == SJVP_FP32; };
     if (!known(in_dtype) || !known(out_dtype)) return SJVP_ERR_DTYPE;
     if (in_dtype != SJVP_FP32 && out_dtype != SJVP_FP32 && in_dtype != out_dtype) return SJVP_ERR_ROTARY;
@@ -397,7 +421,8 @@ int sjvp_rope(int n, const void* const* x, void* const* y, const int64_t* stride
 
     RopeParams p;
     // eight columns per thread need every row start and the second half of a pair 16-byte aligned
-    bool vec = half % 8 == 0 && (D - rot_dim) % 8 == 0 && aligned16(cos) && aligned16(sin) && cs_stride % 4 == 0;
+    bool vec = half % 8 == 0 && (D - rot_dim) % 8 == 0 &&
+               (rot_dim == 0 || (aligned16(cos) && aligned16(sin) && cs_stride % 4 == 0));
     for (int i = 0; i < kRopeMaxTensors; ++i) {
         const int j = i < n ? i : 0;  // unused slots repeat tensor 0 (never dereferenced: grid.y = n)
         if (!x[j] || !y[j]) return SJVP_ERR_NULL;
@@ -462,7 +487,7 @@ const char* sjvp_strerror(int status) {
         case SJVP_ERR_PARTS: return "parts must be SJVP_BWD_ROW, SJVP_BWD_COL or SJVP_BWD_ALL (sjvp_set_row_sum_repair: mode must be SJVP_REPAIR_OFF, _AUTO or _ALWAYS)";
         case SJVP_ERR_SCALE: return "scale must be finite and >= 0 (0 selects 1/sqrt(D))";
         case SJVP_ERR_SCRATCH: return "sjvp_bwd_noalloc: B * H * ceil(Lq/128)*128 exceeds SJVP_NOALLOC_MAX_ROWS, or the static scratch could not be located on this device";
-        case SJVP_ERR_ROTARY: return "rotary embedding: sjvp_rope needs n in 1..4, rot_dim even with 2 <= rot_dim <= D, and no mix of bf16 and fp16; sjvp_fwd_rotary / sjvp_bwd_rotary need D = 64, Lk <= 128, bf16 or fp16 tensors with 16-byte aligned rows, and 16-byte aligned fp32 tables of at least max(Lq, Lk) rows with a row stride that is a multiple of 4";
+        case SJVP_ERR_ROTARY: return "rotary embedding: sjvp_rope needs n in 1..4, rot_dim even with 0 <= rot_dim <= D, and no mix of bf16 and fp16; sjvp_fwd_rotary / sjvp_bwd_rotary need D = 64, Lk <= 128, bf16 or fp16 tensors with 16-byte aligned rows, and 16-byte aligned fp32 tables of at least max(Lq, Lk) rows with a row stride that is a multiple of 4";
         default: return "unknown sjvp status";
     }
 }

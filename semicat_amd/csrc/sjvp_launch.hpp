@@ -4,6 +4,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/sjvp.h"
 #include "sjvp_bwd.hpp"
 #include "sjvp_f32.hpp"
@@ -12,13 +14,47 @@
 namespace sjvp {
 
 // Launch with the status of this launch only (not the thread's sticky last error).
+// A kernel that needs more than 64 KB of LDS has its limit raised first.  K is a function pointer
+// type shared by many kernels, so the (kernel, device) pairs already served are remembered in a small
+// table: the attribute call, which costs host time on every launch otherwise, runs once per pair.
+inline bool lds_limit_raised(const void* kernel, int smem_bytes) {
+    constexpr int kSlots = 512;
+    struct Slot {
+        std::atomic<const void*> kernel{nullptr};
+        std::atomic<int> bytes{0};
+    };
+    static Slot table[kSlots][8];  // open addressing over kernels, by device (devices beyond 8 are not cached)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    Slot* hit = nullptr;
+    if (dev >= 0 && dev < 8) {
+        size_t h = (reinterpret_cast<uintptr_t>(kernel) >> 4) % kSlots;
+        for (int probe = 0; probe < kSlots; ++probe, h = (h + 1) % kSlots) {
+            Slot& s = table[h][dev];
+            const void* cur = s.kernel.load(std::memory_order_acquire);
+            if (cur == kernel) {
+                if (s.bytes.load(std::memory_order_acquire) >= smem_bytes) return true;
+                hit = &s;
+                break;
+            }
+            if (cur == nullptr) {
+                const void* expected = nullptr;
+                if (s.kernel.compare_exchange_strong(expected, kernel, std::memory_order_acq_rel) || expected == kernel) {
+                    hit = &s;
+                    break;
+                }
+            }
+        }
+    }
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes) != hipSuccess) return false;
+    if (hit) hit->bytes.store(smem_bytes, std::memory_order_release);
+    return true;
+}
+
 template <typename K, typename P>
 int launch(K kernel, int grid, int smem_bytes, hipStream_t stream, const P& params, int threads) {
-    if (smem_bytes > 64 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes) != hipSuccess)
-            return SJVP_ERR_LAUNCH;
-    }
+    if (smem_bytes > 64 * 1024 && !lds_limit_raised(reinterpret_cast<const void*>(kernel), smem_bytes))
+        return SJVP_ERR_LAUNCH;
     P copy = params;
     void* args[] = {&copy};
     const hipError_t rc = hipLaunchKernel(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(threads), args,

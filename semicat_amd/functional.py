@@ -38,6 +38,10 @@ from . import kernels
 
 
 AUTOGRAD_WIRING = "fused"  # or "reference"
+# How safe_sdpa_jvp serves float32 callers with bf16 arithmetic: "cast" (default) = the library's
+# multi-tensor cast launches around the 16-bit kernels; "folded" = float32 tensors handed to the
+# kernels, which round as they load and store float32 (SJVP_FP32_BF16, register-staged kernels).
+FP32_CALLERS = "cast"
 
 
 def _has_tangent(t: Tensor) -> bool:
@@ -245,14 +249,22 @@ def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool, arith: Optional[str]
 def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Tensor:
     """``[B,S,H,D]`` wrapper with the reference's dtype policy (functional.py:310-332): inputs that
     are neither bf16 nor fp16 are computed in bfloat16 and the result comes back in their dtype.  For
-    float32 inputs the casts are folded into the kernels (elements are rounded to bf16 as they are
-    loaded, results are stored as float32: no cast kernels run around the op); other dtypes are cast
-    with torch.  ``precise=True`` runs float32 inputs in the library's fp32 mode instead (fp32
-    arithmetic throughout, about 1e-6 against fp64, much slower than the MFMA kernels)."""
+    float32 inputs the casts are the library's own: one launch casts q, k, v (one more their tangents),
+    the 16-bit kernels run, one launch casts the result back (measured faster at every shape than
+    handing the float32 tensors to the kernels, which then run in their register-staged form: see
+    ``FP32_CALLERS``); other dtypes are cast with torch.  ``precise=True`` runs float32 inputs in the
+    library's fp32 mode instead (fp32 arithmetic throughout, about 1e-6 against fp64, much slower
+    than the MFMA kernels)."""
     orig_dtype = q.dtype
     arith = None
-    if orig_dtype == torch.float32 and not precise and AUTOGRAD_WIRING != "reference" \
-            and k.dtype == torch.float32 and v.dtype == torch.float32:
+    fp32_bf16 = orig_dtype == torch.float32 and not precise and AUTOGRAD_WIRING != "reference" \
+        and k.dtype == torch.float32 and v.dtype == torch.float32
+    if fp32_bf16 and FP32_CALLERS == "cast" and q.is_cuda:
+        from .rotary import cast_tensors
+        q, k, v = cast_tensors((q, k, v), torch.bfloat16)
+        y = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), seq_major=True).transpose(1, 2)
+        return cast_tensors(y, orig_dtype)
+    if fp32_bf16 and FP32_CALLERS == "folded":
         arith = "bf16"
     elif orig_dtype != torch.bfloat16 and orig_dtype != torch.float16 and not (precise and orig_dtype == torch.float32):
         q = q.to(torch.bfloat16)
@@ -279,7 +291,7 @@ def safe_sdpa_jvp_rotary(q: Tensor, k: Tensor, v: Tensor, cos: Tensor, sin: Tens
     tangents = [fwAD.unpack_dual(t).tangent for t in (qh, kh, vh)]
     if AUTOGRAD_WIRING != "reference" and kernels.rotary_fusable(
             fwAD.unpack_dual(qh).primal, fwAD.unpack_dual(kh).primal, cos,
-            [fwAD.unpack_dual(vh).primal, *tangents]):
+            [fwAD.unpack_dual(vh).primal, *tangents], sin=sin):
         return _sdpa(qh, kh, vh, seq_major=True, cos=cos, sin=sin).transpose(1, 2)
     from .rotary import apply_rotary
     q, k = apply_rotary((q, k), cos, sin)

@@ -47,21 +47,30 @@ def _rope_args(rope, Lq: int, Lk: int, device):
     return _ptr(cos), _ptr(sin), cos.stride(0), cos.shape[0]
 
 
-def rotary_fusable(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, others: Sequence[torch.Tensor] = ()) -> bool:
+def rotary_fusable(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, others: Sequence[torch.Tensor] = (),
+                   sin: Optional[torch.Tensor] = None) -> bool:
     """Whether ``[B,H,L,D]`` views q, k (and ``others``: v, tangents) can take the attention kernels
     with the rotary embedding folded in: head dimension 64 rotated as a whole, at most 128 keys,
-    16-bit tensors with 16-byte aligned rows, 16-byte aligned fp32 tables."""
+    16-bit tensors with 16-byte aligned rows, and fp32 tables ``[>= max(Lq, Lk), 32]`` on the same
+    device, 16-byte aligned, with unit column stride and equal row strides that are multiples of 4:
+    everything ``_rope_args`` and the C ABI (``check_rotary``) would otherwise reject, so that a
+    caller who asks first never sees their errors and falls back to ``sjvp_rope`` + the plain op."""
     if not q.is_cuda or q.dtype not in (torch.bfloat16, torch.float16) or q.shape[-1] != 64 or k.shape[-2] > 128:
         return False
     # Alignment is judged from the offset into the storage (allocations start on 256-byte boundaries):
     # under torch.func transforms the tensors are wrappers without an address of their own.
-    if cos.shape[-1] != 32 or cos.dtype != torch.float32 or cos.stride(0) % 4 or cos.stride(1) != 1 \
-            or (cos.storage_offset() * 4) % 16:
+    for table in (cos,) if sin is None else (cos, sin):
+        if table.ndim != 2 or table.shape[1] != 32 or table.shape[0] < max(q.shape[-2], k.shape[-2]) \
+                or table.dtype != torch.float32 or table.device != q.device or table.stride(0) % 4 \
+                or table.stride(0) < 32 or table.stride(1) != 1 or (table.storage_offset() * 4) % 16:
+            return False
+    if sin is not None and (sin.shape != cos.shape or sin.stride(0) != cos.stride(0)):
         return False
     for t in (q, k, *others):
         if t is None:
             continue
-        if t.dtype != q.dtype or t.stride(-1) != 1 or (t.storage_offset() * 2) % 16 or any(s % 8 for s in t.stride()[:3]):
+        if t.dtype != q.dtype or t.device != q.device or t.stride(-1) != 1 or (t.storage_offset() * 2) % 16 \
+                or any(s % 8 for s in t.stride()[:3]):
             return False
     return True
 
@@ -411,7 +420,7 @@ def flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, bias=None, causal: bool
 _ROPE_DTYPES = {torch.bfloat16: _lib.SJVP_BF16, torch.float16: _lib.SJVP_FP16, torch.float32: _lib.SJVP_FP32}
 
 
-def rotary_embedding(xs: Sequence[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
+def rotary_embedding(xs: Sequence[torch.Tensor], cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
                      out_dtype: Optional[torch.dtype] = None, inverse: bool = False
                      ) -> Tuple[torch.Tensor, ...]:
     """Rotary position embedding of up to four ``[B,S,H,D]`` tensors of one shape and dtype in one
@@ -419,7 +428,9 @@ def rotary_embedding(xs: Sequence[torch.Tensor], cos: torch.Tensor, sin: torch.T
     flash_attn's ``apply_rotary_emb_torch``; ``cos``/``sin`` are fp32 ``[S, rot/2]`` (any row
     stride).  Inputs may be any views with unit last stride; the results are fresh contiguous
     ``[B,S,H,D]`` tensors of ``out_dtype`` (default: the input dtype).  ``inverse`` applies the
-    inverse rotation (the transpose of the map, which is what back-propagates a cotangent)."""
+    inverse rotation (the transpose of the map, which is what back-propagates a cotangent).
+    ``cos = sin = None``: no rotation, only the cast and the change of layout (one launch for up to
+    four tensors: the casts of functional.py:318-322,330-331 around the op for float32 callers)."""
     xs = tuple(xs)
     if not 1 <= len(xs) <= 4:
         raise ValueError("rotary_embedding takes one to four tensors")
@@ -436,13 +447,16 @@ def rotary_embedding(xs: Sequence[torch.Tensor], cos: torch.Tensor, sin: torch.T
             raise AssertionError("rotary_embedding: all tensors must share shape, dtype and device")
         if x.stride(-1) != 1:
             raise AssertionError("rotary_embedding: the last dimension must have unit stride")
-    half = cos.shape[-1]
-    if cos.shape != sin.shape or cos.ndim != 2 or cos.shape[0] < S or 2 * half > D:
-        raise AssertionError(f"cos/sin must be [>= {S}, rot/2] with rot <= {D}, got {tuple(cos.shape)}")
-    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.stride(1) != 1 or sin.stride(1) != 1 \
-            or cos.stride(0) != sin.stride(0) or cos.device != x0.device or sin.device != x0.device:
-        raise AssertionError("cos/sin must be float32 tensors on the inputs' device with unit column "
-                             "stride and equal row strides")
+    if (cos is None) != (sin is None):
+        raise AssertionError("cos and sin come together")
+    half = 0 if cos is None else cos.shape[-1]
+    if cos is not None:
+        if cos.shape != sin.shape or cos.ndim != 2 or cos.shape[0] < S or 2 * half > D:
+            raise AssertionError(f"cos/sin must be [>= {S}, rot/2] with rot <= {D}, got {tuple(cos.shape)}")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.stride(1) != 1 or sin.stride(1) != 1 \
+                or cos.stride(0) != sin.stride(0) or cos.device != x0.device or sin.device != x0.device:
+            raise AssertionError("cos/sin must be float32 tensors on the inputs' device with unit column "
+                                 "stride and equal row strides")
     ys = tuple(torch.empty((B, S, H, D), device=x0.device, dtype=out_dtype) for _ in xs)
     if B * S * H == 0:
         return ys
@@ -456,7 +470,7 @@ def rotary_embedding(xs: Sequence[torch.Tensor], cos: torch.Tensor, sin: torch.T
     with torch.cuda.device(x0.device):
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.sjvp_rope(n, xp, yp, (ctypes.c_int64 * len(flat))(*flat), _ptr(cos), _ptr(sin),
-                           cos.stride(0), B, H, S, D, 2 * half, _ROPE_DTYPES[x0.dtype],
+                           0 if cos is None else cos.stride(0), B, H, S, D, 2 * half, _ROPE_DTYPES[x0.dtype],
                            _ROPE_DTYPES[out_dtype], 1 if inverse else 0, ctypes.c_void_p(stream))
     _lib.check(rc)
     return ys

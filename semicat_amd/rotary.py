@@ -63,3 +63,15 @@ def apply_rotary(xs, cos: Tensor, sin: Tensor, out_dtype: Optional[torch.dtype] 
     single = isinstance(xs, Tensor)
     ys = RotaryFunction.apply(cos, sin, False, out_dtype, *((xs,) if single else tuple(xs)))
     return ys[0] if single else ys
+
+
+@torch._dynamo.disable
+def cast_tensors(xs, out_dtype: torch.dtype):
+    """Cast a tensor or a tuple of up to four ``[B,S,H,D]`` tensors (views are fine) to ``out_dtype``
+    in ONE launch, into contiguous ``[B,S,H,D]`` results: the rotary function without a rotation, so
+    forward-mode tangents take the same launch and cotangents come back in the inputs' dtype through
+    it.  This is the ``.to(torch.bfloat16)`` / ``.to(orig_dtype)`` pair that
+    semicat/jvp_utils/functional.py:318-322,330-331 puts around the op for float32 callers."""
+    single = isinstance(xs, Tensor)
+    ys = RotaryFunction.apply(None, None, False, out_dtype, *((xs,) if single else tuple(xs)))
+    return ys[0] if single else ys

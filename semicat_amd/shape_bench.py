@@ -1,11 +1,16 @@
 """Step time of the attention-JVP forward + backward at any shape:
-``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16] [--steps K]``.
+``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16|fp32io|fp32cast] [--steps K]``.
 
 The same measurement as the headline benchmark (planned launches through the C ABI on one stream,
 0.3 s of untimed load first, then K timed steps; random q, k, v ~ 0.5 N(0,1), tangents ~ 0.1 N(0,1),
 cotangents ~ N(0,1)), for the shapes the headline benchmark does not cover: longer sequences, other
 head dimensions, keys and queries of different lengths.  Work model 42*B*H*Lq*Lk*D flop per step.
 Prints one JSON line.  A companion measurement, not the headline figure.
+
+``--dtype fp32io`` and ``fp32cast`` time the two ways of serving a float32 caller with bf16 arithmetic
+(the dtype policy of semicat/jvp_utils/functional.py:318-332): the casts folded into the kernels
+(float32 tensors handed over as they are, SJVP_FP32_BF16), or torch casts around the 16-bit kernels
+(six casts in, two out in the forward; two in, six out in the backward).
 """
 from __future__ import annotations
 
@@ -23,7 +28,7 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "H", "L", "D"), default=(128, 12, 256, 64))
     ap.add_argument("--keys", type=int, default=None, help="key/value length (default: L)")
-    ap.add_argument("--dtype", choices=("bf16", "fp16"), default="bf16")
+    ap.add_argument("--dtype", choices=("bf16", "fp16", "fp32io", "fp32cast"), default="bf16")
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     a = ap.parse_args(argv)
@@ -35,8 +40,9 @@ def main(argv=None) -> int:
     torch.cuda.set_device(dev)
     B, H, Lq, D = a.shape
     Lk = a.keys or Lq
-    dt = torch.bfloat16 if a.dtype == "bf16" else torch.float16
-    code = _lib.SJVP_BF16 if a.dtype == "bf16" else _lib.SJVP_FP16
+    fp32 = a.dtype.startswith("fp32")
+    dt = torch.float32 if fp32 else (torch.bfloat16 if a.dtype == "bf16" else torch.float16)
+    code = _lib.SJVP_FP32_BF16 if a.dtype == "fp32io" else (_lib.SJVP_FP16 if a.dtype == "fp16" else _lib.SJVP_BF16)
     g = torch.Generator(device=dev).manual_seed(0)
 
     def rnd(L, s):
@@ -54,9 +60,33 @@ def main(argv=None) -> int:
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        fwd, _ = kernels.plan_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False)
-        bwd, _ = kernels.plan_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads,
-                                       workspace=workspace)
+        if a.dtype == "fp32cast":
+            lo = torch.bfloat16
+            ins16 = [torch.empty_like(t, dtype=lo) for t in (q, k, v, tq, tk, tv)]
+            o16, to16, dO16, dTO16 = (torch.empty_like(q, dtype=lo) for _ in range(4))
+            grads16 = tuple(torch.empty_like(t, dtype=lo) for t in grads)
+            fwd16, _ = kernels.plan_forward(*ins16, o=o16, to=to16, lse=lse, mu=mu, with_li=False)
+            bwd16, _ = kernels.plan_backward(*ins16, o16, to16, lse, mu, dO=dO16, dTO=dTO16, grads=grads16,
+                                             workspace=workspace)
+
+            def fwd():
+                for dst, src in zip(ins16, (q, k, v, tq, tk, tv)):
+                    dst.copy_(src)
+                fwd16()
+                o.copy_(o16)
+                to.copy_(to16)
+
+            def bwd():
+                dO16.copy_(dO)
+                dTO16.copy_(dTO)
+                bwd16()
+                for dst, src in zip(grads, grads16):
+                    dst.copy_(src)
+        else:
+            arith = {"arithmetic": "bf16"} if a.dtype == "fp32io" else {}
+            fwd, _ = kernels.plan_forward(q, k, v, tq, tk, tv, o=o, to=to, lse=lse, mu=mu, with_li=False, **arith)
+            bwd, _ = kernels.plan_backward(q, k, v, tq, tk, tv, o, to, lse, mu, dO=dO, dTO=dTO, grads=grads,
+                                           workspace=workspace, **arith)
         t_ramp = time.perf_counter() + 0.3  # the clocks settle only under sustained load
         while time.perf_counter() < t_ramp:
             for _ in range(5):
@@ -86,8 +116,10 @@ def main(argv=None) -> int:
         bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / n_ev
     unit = float(B) * H * Lq * Lk * D
     print(json.dumps({
-        "workload": f"attention JVP fwd+bwd, B={B} H={H} Lq={Lq} Lk={Lk} D={D}, {a.dtype} in / fp32 acc, "
-                    f"both cotangents",
+        "workload": f"attention JVP fwd+bwd, B={B} H={H} Lq={Lq} Lk={Lk} D={D}, "
+                    + {"fp32io": "fp32 tensors, casts folded into the kernels, bf16 arithmetic",
+                       "fp32cast": "fp32 tensors, torch casts around the bf16 kernels"}.get(
+                           a.dtype, f"{a.dtype} in / fp32 acc") + ", both cotangents",
         "ms_per_step": step_ms, "TFLOPs": 42.0 * unit / (step_ms * 1e-3) / 1e12,
         "fwd_ms": fwd_ms, "fwd_TFLOPs": 12.0 * unit / (fwd_ms * 1e-3) / 1e12,
         "bwd_ms": bwd_ms, "bwd_TFLOPs": 30.0 * unit / (bwd_ms * 1e-3) / 1e12,

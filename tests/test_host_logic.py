@@ -109,9 +109,11 @@ def test_plain_forward_and_backward_without_tangents(monkeypatch):
 
 def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
     """[B,S,H,D] in and out; fp32 inputs are computed in bf16 and come back as fp32
-    (functional.py:318-332) with the casts folded into the launch (the launcher gets the fp32 tensors
-    and arithmetic="bf16"); other dtypes are cast with torch.  Inside the op q,k,v are [B,H,S,D] views
-    with strides (S*H*D, D, H*D, 1)."""
+    (functional.py:318-332): with FP32_CALLERS = "folded" the casts are folded into the launch (the
+    launcher gets the fp32 tensors and arithmetic="bf16"), with the default "cast" the launcher gets
+    bf16 tensors (cast by the library's own kernel on a GPU, by torch on the CPU stand-in of this
+    test); other dtypes are cast with torch.  Inside the op q,k,v are [B,H,S,D] views with strides
+    (S*H*D, D, H*D, 1)."""
     seen = {}
     real = eager_backend.attention_jvp_forward
 
@@ -127,7 +129,11 @@ def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
     g = torch.Generator().manual_seed(0)
     q, k, v, tq, tk, tv = (torch.randn(B, S, H, D, generator=g) for _ in range(6))
     ref = orc.attention_jvp_autograd(*(t.transpose(1, 2) for t in (q, k, v, tq, tk, tv)))
-    for dtype, want in ((torch.float32, (torch.float32, "bf16")), (torch.float64, (torch.bfloat16, None))):
+    assert functional.FP32_CALLERS == "cast"
+    for dtype, want, route in ((torch.float32, (torch.float32, "bf16"), "folded"),
+                               (torch.float32, (torch.bfloat16, None), "cast"),
+                               (torch.float64, (torch.bfloat16, None), "cast")):
+        monkeypatch.setattr(functional, "FP32_CALLERS", route)
         y, ty = torch.func.jvp(functional.safe_sdpa_jvp, tuple(t.to(dtype) for t in (q, k, v)),
                                tuple(t.to(dtype) for t in (tq, tk, tv)))
         assert y.shape == (B, S, H, D) and y.dtype == dtype and ty.dtype == dtype
@@ -260,7 +266,7 @@ def test_c_abi_argument_errors_are_reported_before_any_launch():
     r = lambda **kw: L.sjvp_rope(kw.get("n", 2), kw.get("x", ptrs), ptrs, rs, kw.get("cos", one), one, 32, 1, 1,
                                  kw.get("L", 8), 64, kw.get("rot", 64), kw.get("i", 0), kw.get("o", 0), 0, None)
     assert r(n=0) == _lib.SJVP_ERR_ROTARY and r(n=5) == _lib.SJVP_ERR_ROTARY
-    assert r(rot=63) == _lib.SJVP_ERR_ROTARY and r(rot=66) == _lib.SJVP_ERR_ROTARY and r(rot=0) == _lib.SJVP_ERR_ROTARY
+    assert r(rot=63) == _lib.SJVP_ERR_ROTARY and r(rot=66) == _lib.SJVP_ERR_ROTARY and r(rot=-2) == _lib.SJVP_ERR_ROTARY
     assert r(i=0, o=1) == _lib.SJVP_ERR_ROTARY  # bf16 in, fp16 out
     assert r(i=5) == _lib.SJVP_ERR_DTYPE
     assert r(L=0) == _lib.SJVP_ERR_SHAPE

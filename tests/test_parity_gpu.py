@@ -377,10 +377,14 @@ def test_fp32_tensors_with_bf16_arithmetic(K, mode, B, H, Lq, Lk, D, seq_major):
     assert orc.rel_frobenius(o2.cpu(), ref["O"]) <= TOL_16BIT
 
 
-def test_safe_sdpa_jvp_runs_no_cast_kernels_for_fp32_callers(K):
+@pytest.mark.parametrize("route", ["cast", "folded"])
+def test_safe_sdpa_jvp_runs_no_cast_kernels_for_fp32_callers(K, route, monkeypatch):
     """safe_sdpa_jvp on fp32 [B,S,H,D] tensors under torch.func.jvp and reverse mode: same results as
-    casting to bf16 first, and the only kernels launched are the library's (forward, backward)."""
-    from semicat_amd import safe_sdpa_jvp
+    casting to bf16 first, and the only kernels launched are the library's: by default its
+    multi-tensor cast launches around the 16-bit LDS-DMA kernels ("cast"), or the kernels that take
+    float32 tensors as they are ("folded")."""
+    from semicat_amd import functional, safe_sdpa_jvp
+    monkeypatch.setattr(functional, "FP32_CALLERS", route)
     B, H, L, D = 2, 4, 128, 64
     x32 = orc.make_inputs(B, H, L, L, D, seed=29, tangent_scale=0.1, dtype=torch.float32)
     ref = orc.attention_jvp_autograd(*[x32[n].to(torch.bfloat16) for n in orc.TENSOR_ORDER])
@@ -395,10 +399,27 @@ def test_safe_sdpa_jvp_runs_no_cast_kernels_for_fp32_callers(K):
     print("[kernels launched]", names, flush=True)
     foreign = [n for n in names if "sjvp" not in n and "Memcpy" not in n and "Memset" not in n]
     assert not foreign, foreign
+    if route == "cast":
+        assert any("fwd16_kernel" in n for n in names) and any("bwd_fused16" in n for n in names), names
+        assert sum("rope_kernel" in n for n in names) >= 1
     assert y.dtype == torch.float32 and y.is_contiguous()
     res = {"O": y.detach().transpose(1, 2).cpu(), "TO": ty.detach().transpose(1, 2).cpu(),
            **{n: g_.transpose(1, 2).cpu() for n, g_ in zip(GRADS, grads)}}
     assert_parity(res, ref, TOL_16BIT, label="safe_sdpa_jvp, fp32 caller")
+
+
+def test_few_heads_with_a_long_query_axis_take_the_row_and_column_pair(K):
+    """Two (batch, head) pairs with 600 queries on 128 keys fit the single-launch backward, which would
+    run them on two compute units; the selection hands such problems to the row-owned + column-owned
+    pair, whose row launch spreads the queries over the chip.  Same results to the gate."""
+    from torch.profiler import ProfilerActivity, profile
+    x = orc.make_inputs(1, 2, 600, 128, 64, seed=31, tangent_scale=0.1, dtype=torch.bfloat16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        res = run_hip(K, x)
+    names = [e.key for e in prof.key_averages() if e.device_type == torch.autograd.DeviceType.CUDA]
+    assert any("bwd_row16_kernel" in n for n in names) and not any("bwd_fused16" in n for n in names), names
+    assert_parity(res, ref, TOL_16BIT, label="few heads, long query axis")
 
 
 def test_bitwise_determinism(K):

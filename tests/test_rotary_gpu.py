@@ -186,6 +186,15 @@ def test_shapes_the_folded_rotation_does_not_serve_are_refused(K):
         with pytest.raises(_lib.SjvpError, match="rotary"):
             K.attention_jvp_forward(q, k, k, q, k, k, rope=(cos, sin))
     assert not K.rotary_fusable(z(64).float(), z(64).float(), cos)
+    # tables the launchers would reject are refused here too, so that callers fall back instead of raising
+    q = z(64)
+    assert K.rotary_fusable(q, q, cos, sin=sin)
+    assert not K.rotary_fusable(q, q, cos[:32], sin=sin[:32])                 # fewer rows than positions
+    assert not K.rotary_fusable(q, q, cos, sin=sin.double())                   # sin of another dtype
+    assert not K.rotary_fusable(q, q, cos, sin=sin.cpu())                      # sin on another device
+    assert not K.rotary_fusable(q, q, cos, sin=torch.zeros(256, 64, device="cuda")[:, ::2])  # strided columns
+    assert not K.rotary_fusable(q, q, cos.reshape(-1)[1:1 + 255 * 32].view(255, 32))  # misaligned table
+    assert not K.rotary_fusable(q, q, cos[None])                               # not two-dimensional
 
 
 def test_network_block_issues_no_rotary_launch_at_sequence_128():

@@ -34,7 +34,7 @@ def _call(lib, entry, d, o, to, lse, mu, shape, with_workspace):
 
 @pytest.mark.parametrize("shapes", [
     [(2, 3, 300, 260, 64), (1, 2, 130, 200, 64)],    # row + column pair, then a smaller problem
-    [(1, 2, 200, 150, 128), (2, 2, 128, 128, 64)],   # D = 128 (split column launches), then the single launch
+    [(1, 2, 200, 150, 128), (2, 2, 128, 128, 64)],   # D = 128 (paired-wave column launch), then the single launch
 ])
 def test_noalloc_backward_equals_the_workspace_entry_point(shapes):
     assert torch.cuda.is_available(), "this test needs the MI355X"
@@ -60,6 +60,56 @@ def test_noalloc_backward_equals_the_workspace_entry_point(shapes):
         torch.cuda.synchronize()
         for a, b in zip(via, want):
             assert torch.equal(a, b)
+
+
+def test_noalloc_backward_replays_in_a_captured_graph():
+    """The use the entry point is for: captured in a HIP graph (its first call on the device made
+    outside the capture, which is when the array's address is looked up), replayed three times with
+    fresh inputs copied in and eager work between the replays; every replay equals the eager sjvp_bwd
+    result bit for bit."""
+    from semicat_amd import kernels
+    B, H, Lq, Lk, D = 2, 3, 260, 200, 64  # the row + column pair: the launches that use the scratch
+    names = orc.TENSOR_ORDER
+    sets = [orc.make_inputs(B, H, Lq, Lk, D, seed=60 + i, tangent_scale=0.3, dtype=torch.bfloat16) for i in range(3)]
+    d = {n: torch.empty_like(sets[0][n], device="cuda") for n in names}
+    o, to = torch.empty_like(d["q"]), torch.empty_like(d["q"])
+    lse = torch.empty((B, H, kernels.stat_rows(Lq)), device="cuda", dtype=torch.float32)
+    mu = torch.empty_like(lse)
+    grads = tuple(torch.empty_like(d[n]) for n in ("q", "k", "v", "tq", "tk", "tv"))
+
+    def load(i):
+        for n in names:
+            d[n].copy_(sets[i][n])
+
+    def step(static):
+        kernels.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o=o, to=to, lse=lse, mu=mu,
+                                      with_li=False)
+        kernels.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                       dO=d["dO"], dTO=d["dTO"], grads=grads, static_scratch=static)
+
+    eager = []
+    for i in range(3):
+        load(i)
+        step(False)  # sjvp_bwd with a workspace of its own
+        torch.cuda.synchronize()
+        eager.append([t.clone() for t in grads])
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        load(0)
+        step(True)  # first call on the device, outside the capture
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step(True)
+        for i in (1, 2, 0):
+            load(i)
+            for t in grads:
+                t.zero_()
+            stream.synchronize()
+            graph.replay()
+            stream.synchronize()
+            for n, got, want in zip(GRADS, grads, eager[i]):
+                assert torch.equal(got, want), f"replay on input set {i}: {n} differs from the eager sjvp_bwd"
 
 
 def test_noalloc_backward_rejects_problems_beyond_its_scratch():
