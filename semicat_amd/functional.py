@@ -38,10 +38,16 @@ from . import kernels
 
 
 AUTOGRAD_WIRING = "fused"  # or "reference"
-# How safe_sdpa_jvp serves float32 callers with bf16 arithmetic: "cast" (default) = the library's
-# multi-tensor cast launches around the 16-bit kernels; "folded" = float32 tensors handed to the
-# kernels, which round as they load and store float32 (SJVP_FP32_BF16, register-staged kernels).
-FP32_CALLERS = "cast"
+# How safe_sdpa_jvp serves float32 callers with bf16 arithmetic (functional.py:318-332):
+#   "torch"   (default) torch casts around the 16-bit LDS-DMA kernels, as the reference does;
+#   "library" the library's multi-tensor cast launches around them (half the launches, no kernel that is
+#             not the library's own; the same speed on large problems, more host time on small ones);
+#   "folded"  the float32 tensors handed to the kernels, which round as they load and store float32
+#             (SJVP_FP32_BF16: register-staged kernels, no cast at all, but 1.1 to 2.4 times slower).
+# Measured on an MI355X, forward + backward in microseconds, 16-bit callers / torch / library / folded:
+#   B=64 H=12 L=128 D=64: 70 / 218 / 207 / 244;  B=128 H=12 L=256: 502 / 936 / 934 / 1609;
+#   B=8 H=16 L=1024: 514 / 687 / 668 / 1614;  B=2 H=4 L=256 (host-bound): 41 / 76 / 212 / 86.
+FP32_CALLERS = "torch"
 
 
 def _has_tangent(t: Tensor) -> bool:
@@ -248,18 +254,17 @@ def _sdpa(q: Tensor, k: Tensor, v: Tensor, seq_major: bool, arith: Optional[str]
 
 def safe_sdpa_jvp(q: Tensor, k: Tensor, v: Tensor, precise: bool = False) -> Tensor:
     """``[B,S,H,D]`` wrapper with the reference's dtype policy (functional.py:310-332): inputs that
-    are neither bf16 nor fp16 are computed in bfloat16 and the result comes back in their dtype.  For
-    float32 inputs the casts are the library's own: one launch casts q, k, v (one more their tangents),
-    the 16-bit kernels run, one launch casts the result back (measured faster at every shape than
-    handing the float32 tensors to the kernels, which then run in their register-staged form: see
-    ``FP32_CALLERS``); other dtypes are cast with torch.  ``precise=True`` runs float32 inputs in the
+    are neither bf16 nor fp16 are computed in bfloat16 and the result comes back in their dtype, cast
+    with torch as in the reference; for float32 inputs ``FP32_CALLERS`` selects two other routes (the
+    library's own cast launches, or float32 tensors handed to the kernels as they are), both measured
+    slower or equal (figures beside ``FP32_CALLERS``).  ``precise=True`` runs float32 inputs in the
     library's fp32 mode instead (fp32 arithmetic throughout, about 1e-6 against fp64, much slower
     than the MFMA kernels)."""
     orig_dtype = q.dtype
     arith = None
     fp32_bf16 = orig_dtype == torch.float32 and not precise and AUTOGRAD_WIRING != "reference" \
         and k.dtype == torch.float32 and v.dtype == torch.float32
-    if fp32_bf16 and FP32_CALLERS == "cast" and q.is_cuda:
+    if fp32_bf16 and FP32_CALLERS == "library" and q.is_cuda:
         from .rotary import cast_tensors
         q, k, v = cast_tensors((q, k, v), torch.bfloat16)
         y = _sdpa(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), seq_major=True).transpose(1, 2)

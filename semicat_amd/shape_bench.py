@@ -1,5 +1,5 @@
 """Step time of the attention-JVP forward + backward at any shape:
-``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16|fp32io|fp32cast] [--steps K]``.
+``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16|fp32io|fp32cast|fp32lib] [--steps K]``.
 
 The same measurement as the headline benchmark (planned launches through the C ABI on one stream,
 0.3 s of untimed load first, then K timed steps; random q, k, v ~ 0.5 N(0,1), tangents ~ 0.1 N(0,1),
@@ -10,7 +10,8 @@ Prints one JSON line.  A companion measurement, not the headline figure.
 ``--dtype fp32io`` and ``fp32cast`` time the two ways of serving a float32 caller with bf16 arithmetic
 (the dtype policy of semicat/jvp_utils/functional.py:318-332): the casts folded into the kernels
 (float32 tensors handed over as they are, SJVP_FP32_BF16), or torch casts around the 16-bit kernels
-(six casts in, two out in the forward; two in, six out in the backward).
+(six casts in, two out in the forward; two in, six out in the backward), or (``fp32lib``) the
+library's own multi-tensor cast launches around them, which is what ``safe_sdpa_jvp`` does.
 """
 from __future__ import annotations
 
@@ -28,7 +29,7 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "H", "L", "D"), default=(128, 12, 256, 64))
     ap.add_argument("--keys", type=int, default=None, help="key/value length (default: L)")
-    ap.add_argument("--dtype", choices=("bf16", "fp16", "fp32io", "fp32cast"), default="bf16")
+    ap.add_argument("--dtype", choices=("bf16", "fp16", "fp32io", "fp32cast", "fp32lib"), default="bf16")
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     a = ap.parse_args(argv)
@@ -60,7 +61,28 @@ def main(argv=None) -> int:
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        if a.dtype == "fp32cast":
+        if a.dtype == "fp32lib":
+            # the route safe_sdpa_jvp takes for float32 callers: the library's multi-tensor cast launches
+            # ([B,S,H,D] views in and out) around the 16-bit kernels
+            lo = torch.bfloat16
+            bshd = lambda t: t.transpose(1, 2)
+            cast = lambda ts, dt_: tuple(bshd(y) for y in kernels.rotary_embedding([bshd(t) for t in ts], None, None,
+                                                                                   out_dtype=dt_))
+            state = {}
+
+            def fwd():
+                a16 = cast((q, k, v), lo) + cast((tq, tk, tv), lo)
+                o16, to16, _, _, _ = kernels.attention_jvp_forward(*a16, lse=lse, mu=mu, with_li=False)
+                state["saved"] = (a16, o16, to16)
+                state["out"] = cast((o16, to16), torch.float32)
+
+            def bwd():
+                a16, o16, to16 = state["saved"]
+                d16 = cast((dO, dTO), lo)
+                g16 = kernels.attention_jvp_backward(*a16, o16, to16, lse, mu, dO=d16[0], dTO=d16[1],
+                                                     workspace=workspace)
+                state["grads"] = cast(g16[:3], torch.float32) + cast(g16[3:], torch.float32)
+        elif a.dtype == "fp32cast":
             lo = torch.bfloat16
             ins16 = [torch.empty_like(t, dtype=lo) for t in (q, k, v, tq, tk, tv)]
             o16, to16, dO16, dTO16 = (torch.empty_like(q, dtype=lo) for _ in range(4))
@@ -118,6 +140,7 @@ def main(argv=None) -> int:
     print(json.dumps({
         "workload": f"attention JVP fwd+bwd, B={B} H={H} Lq={Lq} Lk={Lk} D={D}, "
                     + {"fp32io": "fp32 tensors, casts folded into the kernels, bf16 arithmetic",
+                       "fp32lib": "fp32 tensors, the library's cast launches around the bf16 kernels",
                        "fp32cast": "fp32 tensors, torch casts around the bf16 kernels"}.get(
                            a.dtype, f"{a.dtype} in / fp32 acc") + ", both cotangents",
         "ms_per_step": step_ms, "TFLOPs": 42.0 * unit / (step_ms * 1e-3) / 1e12,

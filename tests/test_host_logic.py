@@ -110,9 +110,8 @@ def test_plain_forward_and_backward_without_tangents(monkeypatch):
 def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
     """[B,S,H,D] in and out; fp32 inputs are computed in bf16 and come back as fp32
     (functional.py:318-332): with FP32_CALLERS = "folded" the casts are folded into the launch (the
-    launcher gets the fp32 tensors and arithmetic="bf16"), with the default "cast" the launcher gets
-    bf16 tensors (cast by the library's own kernel on a GPU, by torch on the CPU stand-in of this
-    test); other dtypes are cast with torch.  Inside the op q,k,v are [B,H,S,D] views with strides
+    launcher gets the fp32 tensors and arithmetic="bf16"), with the default "torch" the launcher gets
+    bf16 tensors; other dtypes are cast with torch.  Inside the op q,k,v are [B,H,S,D] views with strides
     (S*H*D, D, H*D, 1)."""
     seen = {}
     real = eager_backend.attention_jvp_forward
@@ -129,10 +128,10 @@ def test_safe_sdpa_jvp_layout_and_dtype(monkeypatch):
     g = torch.Generator().manual_seed(0)
     q, k, v, tq, tk, tv = (torch.randn(B, S, H, D, generator=g) for _ in range(6))
     ref = orc.attention_jvp_autograd(*(t.transpose(1, 2) for t in (q, k, v, tq, tk, tv)))
-    assert functional.FP32_CALLERS == "cast"
+    assert functional.FP32_CALLERS == "torch"
     for dtype, want, route in ((torch.float32, (torch.float32, "bf16"), "folded"),
-                               (torch.float32, (torch.bfloat16, None), "cast"),
-                               (torch.float64, (torch.bfloat16, None), "cast")):
+                               (torch.float32, (torch.bfloat16, None), "torch"),
+                               (torch.float64, (torch.bfloat16, None), "torch")):
         monkeypatch.setattr(functional, "FP32_CALLERS", route)
         y, ty = torch.func.jvp(functional.safe_sdpa_jvp, tuple(t.to(dtype) for t in (q, k, v)),
                                tuple(t.to(dtype) for t in (tq, tk, tv)))
