@@ -147,7 +147,7 @@ int sjvp_bwd_rotary(const void* q, const void* k, const void* v, const void* tq,
  * caller buffer.  It has no counterpart in the reference; it is for callers that cannot allocate
  * device memory around the call: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc.  The call allocates and frees nothing (neither does the rest of this library).
- *   - Limit: B * H * ceil(Lq/128)*128 <= SJVP_NOALLOC_MAX_ROWS (1 Mi statistic rows, 12 MiB of
+ *   - Limit: B * H * ceil(Lq/128)*128 <= SJVP_NOALLOC_MAX_ROWS (1 Mi statistic rows, 12.1 MiB of
  *     device memory that every GPU the library runs on holds until the process ends); larger
  *     problems return SJVP_ERR_SCRATCH and must use sjvp_bwd().
  *   - Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two streams,
@@ -170,14 +170,18 @@ int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq
  * (flash_jvp_backward.py:2012-2290) and delta from the 16-bit output (flash_attn_triton.py:526-617).
  * This library takes all of them from the 16-bit outputs o, to, which costs no pass, and the
  * row-owned launch then measures what the rounding of o, to left in them (the sums over the keys of
- * dS_dot and of dS, zero in exact arithmetic): it hands the column-owned launch the corrected sums,
- * and repairs its own dq, dtq with one more pass over k (, tk) of the workgroups that need it.
- *   SJVP_REPAIR_OFF     never run the second pass (dk, dtk still get the corrected sums)
- *   SJVP_REPAIR_AUTO    (default) second pass where a row's residue exceeds the rounding of the tiles it
- *                       is spread over: sharp attention rows, gradients formed by cancellation
- *   SJVP_REPAIR_ALWAYS  second pass everywhere, and the row + column pair also for the shapes that
- *                       would take the single launch, whose row sums stay those of the 16-bit outputs
- *                       (not with sjvp_bwd_rotary): every gradient as accurate as the reference's form
+ * dS_dot and of dS, zero in exact arithmetic): it hands the column-owned launch the corrected sums
+ * (= the reference's sums), and a second launch of the row-owned kernel recomputes dq, dtq with them
+ * for the workgroups that ask for it.
+ *   SJVP_REPAIR_OFF     no second launch (dk, dtk still get the corrected sums)
+ *   SJVP_REPAIR_AUTO    (default) the second launch runs the workgroups in which a row's residue exceeds
+ *                       the rounding of the tiles it is spread over (sharp attention rows, gradients
+ *                       formed by cancellation); the others leave at once
+ *   SJVP_REPAIR_ALWAYS  the first launch only measures, the second computes every row with the
+ *                       corrected sums (the reference's preprocess + backward structure), and the row +
+ *                       column pair is taken also for the shapes that would take the single launch,
+ *                       whose row sums stay those of the 16-bit outputs (not with sjvp_bwd_rotary):
+ *                       every gradient is formed as the reference forms it
  * Process-wide; returns the previous mode, or SJVP_ERR_PARTS for an unknown one.  Calls already
  * enqueued are not affected.
  */
@@ -186,7 +190,8 @@ int sjvp_set_row_sum_repair(int mode);
 
 /* Bytes of caller-provided device scratch sjvp_bwd needs: lse in log2 units and the row sums sum_4
  * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,
- * flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990). */
+ * flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990), 12 bytes per statistic row, and one
+ * 4-byte flag per 64 rows (which row-owned workgroups take the second launch of the repair below). */
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
 
 /*

@@ -343,9 +343,9 @@ def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, s
 
     ``repaired`` (with ``sums_from_outputs``) models what the row-owned + column-owned kernels do about
     it: the residues ``rho4 = sum_j dS_dot``, ``rho7 = sum_j dS`` (zero with exact sums) are measured on
-    the unrounded tiles; the key side is formed with the corrected sums ``s4 + rho4``, ``s7d + rho7``; the
-    query side keeps the tiles formed with the rounded sums and subtracts ``s rho4 (P K)`` from dq_dot
-    and ``s (rho4 ((P*N) K + P K_dot) + rho7 (P K))`` from dq, with P and P*N rounded to ``dtype``.
+    the unrounded tiles formed with the rounded sums, and every gradient is then formed with the
+    corrected sums ``s4 + rho4``, ``s7d + rho7`` (the column pass always, the row pass in its second
+    launch).  In exact arithmetic the corrected sums are the sums of the second form.
     Returns dq, dk, dtq, dtk."""
     r = lambda x: _round_to(x, dtype)
     q, k, v, tq, tk, tv, dOn, G = (r(_f64(x).numpy()) for x in (q, k, v, tq, tk, tv, dO, dTO))
@@ -367,15 +367,10 @@ def row_sum_rounding_model(q, k, v, tq, tk, tv, dO, dTO, dtype=torch.bfloat16, s
     dTS = P * (W - s4)
     dS = dTS * N + P * (XY - s7d)
     if repaired and sums_from_outputs:
-        rho4, rho7 = dTS.sum(-1, keepdims=True), dS.sum(-1, keepdims=True)
-        dTSc = P * (W - (s4 + rho4))
-        dSc = r(dTSc * N + P * (XY - (s7d + rho7)))
-        dTSc = r(dTSc)
-        dTSr, dSr, Pr, PNr = r(dTS), r(dS), r(P), r(P * N)
-        PK = Pr @ k
-        return {"dq": r(s * (dSr @ k + dTSr @ tk - rho4 * (PNr @ k + Pr @ tk) - rho7 * PK)),
-                "dk": r(s * (T(dSc) @ q + T(dTSc) @ tq)),
-                "dtq": r(s * (dTSr @ k - rho4 * PK)), "dtk": r(s * T(dTSc) @ q)}
+        s4 = s4 + dTS.sum(-1, keepdims=True)
+        s7d = s7d + dS.sum(-1, keepdims=True)
+        dTS = P * (W - s4)
+        dS = dTS * N + P * (XY - s7d)
     dS = r(dS)
     dTS = r(dTS)
     return {"dq": r(s * (dS @ k + dTS @ tk)), "dk": r(s * (T(dS) @ q + T(dTS) @ tq)),

@@ -122,7 +122,8 @@ int check_bwd(int parts, const BwdTensors& t, int B, int H, int Lq, int Lk, int 
     return check_common(B, H, Lq, Lk, D, dtype, scale);
 }
 
-// Launches of the backward on a validated problem; `ws` holds 3 * B * H * Lr floats.
+// Launches of the backward on a validated problem; `ws` holds sjvp_bwd_workspace_bytes(): 3 * B * H * Lr
+// floats and, behind them, B * H * Lr / 64 flags.
 int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int Lk, int D,
             const int64_t* strides, float scale, int dtype, void* stream,
             RopeTables rope = RopeTables{nullptr, nullptr, 0, 0}) {
@@ -201,6 +202,7 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
     p.lse2 = ws;
     p.s4 = p.lse2 + (size_t)B * H * p.Lr;
     p.s7d = p.s4 + (size_t)B * H * p.Lr;
+    p.flags = reinterpret_cast<int*>(p.s7d + (size_t)B * H * p.Lr);  // one per 64 statistic rows
     p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
     p.rope = rope;
@@ -215,11 +217,12 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
 }
 
 // Scratch of sjvp_bwd_noalloc(): the backward's workspace (lse in log2 units and the two row sums,
-// 3 floats per statistic row) for up to SJVP_NOALLOC_MAX_ROWS rows, resident in every GPU the library
+// 3 floats per statistic row, and one flag per 64 rows) for up to SJVP_NOALLOC_MAX_ROWS rows, resident in every GPU the library
 // runs on from the moment its code is loaded until the process ends.  In host code the array's name
 // is only a handle for hipGetSymbolAddress(); its device address differs from GPU to GPU and is
 // looked up once per device, with that device current.
-static __device__ __align__(256) __attribute__((used)) float scratch[3 * (size_t)SJVP_NOALLOC_MAX_ROWS];
+static __device__ __align__(256) __attribute__((used)) float scratch[3 * (size_t)SJVP_NOALLOC_MAX_ROWS +
+                                                                    SJVP_NOALLOC_MAX_ROWS / 64];
 
 std::mutex g_scratch_mutex;
 float* g_scratch_ptr[kMaxDevices] = {};
@@ -347,7 +350,9 @@ size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype) 
     (void)D;
     (void)dtype;
     if (B < 1 || H < 1 || Lq < 1) return 0;
-    return (size_t)3 * (size_t)B * (size_t)H * (size_t)round_up(Lq, 128) * sizeof(float);
+    // three floats per statistic row (lse in log2 units, the two row sums) and one flag per 64 rows
+    const size_t rows = (size_t)B * (size_t)H * (size_t)round_up(Lq, 128);
+    return 3 * rows * sizeof(float) + rows / 64 * sizeof(int);
 }
 
 int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const void* tk,

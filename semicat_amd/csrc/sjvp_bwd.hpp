@@ -40,7 +40,8 @@ struct BwdParams {
     float scale;
     int vec;
     RopeTables rope;  // q, k (and tangents) are rotated as they are loaded, their gradients rotated back
-    int rowfix;        // repair of dQ, dQ_dot for the residues of the row sums: 0 never, 1 where needed, 2 always
+    int* flags;        // workspace [B*H][Lr/64]: row-owned workgroups whose rows need the second launch
+    int rowfix;        // second launch of the row-owned kernel: 0 never, 1 flagged workgroups, 2 always
     float rowfix_tau;  // a residue counts once it exceeds this fraction of the row's absolute tile sum
 };
 
@@ -55,8 +56,13 @@ struct RowSmem {
     static constexpr int bytes = slot * (int)sizeof(elem_t);
 };
 
-template <typename T, int HD, bool HAS_DO, bool HAS_G, bool F32IO = false>
+// PASS: 0 the first (or only) launch; 1 the first launch of the "always" mode, which only measures the
+// residues; 2 the second launch of the residue repair described in sjvp_bwd16x.hpp (sums from the
+// workspace; workgroups that were not flagged leave at once).
+template <typename T, int HD, bool HAS_DO, bool HAS_G, bool F32IO = false, int PASS = 0>
 __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p) {
+    constexpr bool SECOND = PASS == 2;   // second launch: sums from the workspace, flagged workgroups only
+    constexpr bool MEASURE = PASS == 1;  // first launch of "always": residues and sums only, no gradients
     extern __shared__ __align__(16) unsigned char smem_raw[];
     elem_t* stage = reinterpret_cast<elem_t*>(smem_raw);
 
@@ -76,6 +82,9 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     const int qrow = qb * kOwned + wave * 32 + x;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (qb * kOwned + wave * 32) < p.Lq;
+    if constexpr (SECOND) {
+        if (p.rowfix == 1 && p.flags[blockIdx.x] == 0) return;  // nothing to repair in this workgroup's rows
+    }
 
     u32x4 qB[KC], tqB[KC], gB[KC], doB[KC], oR[KC], toR[KC];
     float lse2 = 0.f, mu = 0.f;
@@ -86,7 +95,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
             qB[c] = load8_io<T, F32IO>(qp, 16 * c + 8 * hf, p.D, qvalid, vec);
-            oR[c] = load8_io<T, F32IO>(op, 16 * c + 8 * hf, p.D, qvalid, vec);
+            if constexpr (!SECOND) oR[c] = load8_io<T, F32IO>(op, 16 * c + 8 * hf, p.D, qvalid, vec);
         }
         if constexpr (HAS_G) {
             const elem_t* tqp = p.tq.head(b, h) + (int64_t)qrow * p.tq.sl;
@@ -96,7 +105,7 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
             for (int c = 0; c < KC; ++c) {
                 tqB[c] = load8_io<T, F32IO>(tqp, 16 * c + 8 * hf, p.D, qvalid, vec);
                 gB[c] = load8_io<T, F32IO>(gp, 16 * c + 8 * hf, p.D, qvalid, vec);
-                toR[c] = load8_io<T, F32IO>(top, 16 * c + 8 * hf, p.D, qvalid, vec);
+                if constexpr (!SECOND) toR[c] = load8_io<T, F32IO>(top, 16 * c + 8 * hf, p.D, qvalid, vec);
             }
         }
         if constexpr (HAS_DO) {
@@ -137,7 +146,13 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         s4 += other_half(s4);
         s7d += other_half(s7d);
     };
-    row_sums();
+    if constexpr (SECOND) {
+        // the corrected sums the first launch left in the workspace
+        s4 = p.s4[so];
+        s7d = p.s7d[so];
+    } else {
+        row_sums();
+    }
     const elem_t* kg = p.k.head(b, h);
     const elem_t* vg = p.v.head(b, h);
     const elem_t* tkg = HAS_G ? p.tk.head(b, h) : nullptr;
@@ -160,6 +175,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         dq[t] = f32x16{0};
         if constexpr (HAS_G) dtq[t] = f32x16{0};
     }
+    // First launch: this lane's part of sum_j dS_dot_ij and sum_j dS_ij, which are zero with exact row
+    // sums and equal minus the rounding error of s4, s7d otherwise, and of their absolute sums (sampled
+    // on every fourth key: they only set the scale of a threshold).
+    float r4 = 0.f, r7 = 0.f, a4 = 0.f, a7 = 0.f;
 
     auto compute = [&](int k0, auto ragged_tag) {
         constexpr bool RAGGED = decltype(ragged_tag)::value;
@@ -196,10 +215,19 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
                 const float dts = pj * (w[j] - s4);
                 w[j] = dts;
                 xy[j] = fmaf(dts, n, pj * (xy[j] - s7d));
+                if constexpr (!SECOND) {
+                    r4 += dts;
+                    if ((j & 3) == 0) a4 += fabsf(dts);
+                }
             } else {
                 xy[j] = pj * (xy[j] - s7d);
             }
+            if constexpr (!SECOND) {
+                r7 += xy[j];
+                if ((j & 3) == 0) a7 += fabsf(xy[j]);
+            }
         }
+        if constexpr (MEASURE) return;  // a launch that only measures the residues
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
             const u32x4 dsB = pack_b<T>(xy, c);
@@ -219,11 +247,10 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
     };
 
     const int n = (p.Lk + kStageRows - 1) / kStageRows;
-    if (hf == 0) {  // every row below Lr is written (zeros beyond Lq): the column-owned kernel, which
-                    // runs after this one, stages 32-row groups
-        p.lse2[so] = lse2;
-        p.s4[so] = s4;
-        p.s7d[so] = s7d;
+    // every row below Lr gets its workspace entries (zeros beyond Lq): the column-owned kernel, which
+    // runs after this one, stages 32-row groups
+    if constexpr (!SECOND) {
+        if (hf == 0) p.lse2[so] = lse2;
     }
     for (int i = 0; i < n; ++i) {
         workgroup_barrier();  // the previous stage is fully consumed
@@ -233,6 +260,25 @@ __global__ __launch_bounds__(kThreads, 1) void bwd_row_kernel(const BwdParams p)
         const int k0 = i * kStageRows;
         if (k0 + kStageRows > p.Lk) compute(k0, std::true_type{});
         else compute(k0, std::false_type{});
+    }
+    if constexpr (!SECOND) {
+        // the residues of the row sums: corrected sums for the column-owned kernel and for the second
+        // launch, which the workgroup asks for where a residue is not small against the rounding of the
+        // tiles it is spread over
+        r4 += other_half(r4);
+        r7 += other_half(r7);
+        a4 = 4.0f * (a4 + other_half(a4));
+        a7 = 4.0f * (a7 + other_half(a7));
+        if (hf == 0) {
+            p.s4[so] = s4 + r4;
+            p.s7d[so] = s7d + r7;
+        }
+        const bool wanted = qvalid && (fabsf(r4) > p.rowfix_tau * a4 || fabsf(r7) > p.rowfix_tau * a7);
+        if (p.rowfix == 1) {
+            const bool any = workgroup_barrier_or(wanted);
+            if (tid == 0) p.flags[blockIdx.x] = any ? 1 : 0;
+        }
+        if constexpr (MEASURE) return;  // the second launch writes dQ, dQ_dot
     }
     if (!qvalid) return;
     elem_t* dqrow = p.dq.head(b, h) + (int64_t)qrow * p.dq.sl;

@@ -14,14 +14,15 @@
 // sums, sum_j dS_dot_ij = sum_j dS_ij = 0 for every query i; with the rounded ones the sums over the
 // keys come out as rho4 = -e4 and rho7 = -e7.  A wave owns whole query rows, so it accumulates both
 // residues in fp32 beside its tiles (per-lane adds) and
-//   - leaves the corrected sums s4' + rho4, s7d' + rho7 in the workspace: the column-owned kernel
-//     works with sums as accurate as the ones the reference's preprocess kernel forms from the
-//     probabilities (semicat/jvp_utils/flash_jvp_backward.py:2266-2287);
-//   - repairs its own dQ_dot, dQ, which were accumulated with the rounded sums and therefore carry
-//     -s rho4 (P K) and -s (rho4 ((P*N) K + P K_dot) + rho7 (P K)): where a residue is not small against
-//     the row's |dS_dot| / |dS| mass (sharp rows, gradients formed by cancellation), the workgroup
-//     streams K (, K_dot) a second time, forms P K and (P*N) K + P K_dot, and subtracts
-//     (BwdParams::rowfix: 0 never, 1 where the residues call for it, 2 always).
+//   - leaves the corrected sums s4' + rho4 = sum_j P W, s7d' + rho7 = sum_j P (N W + XY) in the
+//     workspace: the column-owned kernel works with the sums the reference's preprocess kernel forms
+//     from the probabilities (semicat/jvp_utils/flash_jvp_backward.py:2266-2287);
+//   - flags its workgroup where a residue is not small against the row's |dS_dot| / |dS| mass (sharp
+//     rows, gradients formed by cancellation).  A second launch of the same kernel (PASS = 2) runs the
+//     flagged workgroups again with the corrected sums, so that their dQ, dQ_dot are formed from tiles
+//     that were rounded without the residue in them; the others leave at once.
+// BwdParams::rowfix: 0 no second launch; 1 as described; 2 every workgroup runs twice and the first
+// launch (PASS = 1) only measures (the reference's preprocess + backward structure).
 #pragma once
 #include "sjvp_bwd.hpp"
 #include "sjvp_w16.hpp"
@@ -60,8 +61,10 @@ struct Row16Smem {
     static_assert(R * slot >= kXWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC>
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC, int PASS = 0>
 __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdParams p) {
+    constexpr bool SECOND = PASS == 2;   // second launch: sums from the workspace, flagged workgroups only
+    constexpr bool MEASURE = PASS == 1;  // first launch of "always": residues and sums only, no gradients
     extern __shared__ __align__(16) unsigned char smem_raw[];
     using SM = Row16Smem<HD, R, HAS_G>;
     elem_t* ring = reinterpret_cast<elem_t*>(smem_raw);
@@ -85,6 +88,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     const int qrow = q0 + wave * 16 + n;
     const bool qvalid = qrow < p.Lq;
     const bool wave_active = (q0 + wave * 16) < p.Lq;
+    if constexpr (SECOND) {
+        if (p.rowfix == 1 && p.flags[bid] == 0) return;  // nothing to repair in this workgroup's rows
+    }
 
     // the ring first, so that the copies stream while the own rows are fetched
     using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
@@ -107,33 +113,41 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     // lane's 16-byte pieces, combined over the four lanes of a query
     u32x4 qB[KC], tqB[KC], gB[KC], doB[KC];
     float s4 = 0.f, s7d = 0.f;
+    const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
     {
         u32x4 oR[KC], toR[KC];
         load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
-        load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
+        if constexpr (!SECOND) load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
         if constexpr (HAS_G) {
             load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
             load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
-            load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
+            if constexpr (!SECOND) load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
         }
         if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
+        if constexpr (SECOND) {
+            // the corrected sums the first launch left in the workspace
+            s4 = p.s4[so];
+            s7d = p.s7d[so];
+        } else {
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-            if constexpr (HAS_G) {
-                s4 += dot8<T>(gB[c], oR[c]);
-                s7d += dot8<T>(gB[c], toR[c]);
+            for (int c = 0; c < KC; ++c) {
+                if constexpr (HAS_G) {
+                    s4 += dot8<T>(gB[c], oR[c]);
+                    s7d += dot8<T>(gB[c], toR[c]);
+                }
+                if constexpr (HAS_DO) s7d += dot8<T>(doB[c], oR[c]);
             }
-            if constexpr (HAS_DO) s7d += dot8<T>(doB[c], oR[c]);
+            s4 = group_sum(s4);
+            s7d = group_sum(s7d);
         }
-        s4 = group_sum(s4);
-        s7d = group_sum(s7d);
     }
-    const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
     const float lse2 = p.lse[so] * kLog2e;
     const float mu = HAS_G ? p.mu[so] : 0.f;
     // every row below Lr gets its workspace entries (zeros beyond Lq except lse2, which is finite): the
     // column-owned kernel, which runs after this one, stages 32-row groups
-    if (g == 0) p.lse2[so] = lse2;
+    if constexpr (!SECOND) {
+        if (g == 0) p.lse2[so] = lse2;
+    }
     const float sl2 = p.scale * kLog2e;
     f32x4 dq[DT], dtq[DT];
 #pragma unroll
@@ -141,8 +155,8 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         dq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         dtq[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    // this lane's part of sum_j dS_dot_ij, sum_j dS_ij (zero in exact arithmetic), and of their absolute
-    // sums, which only set the scale of a threshold and are sampled on every fourth key
+    // First launch: this lane's part of sum_j dS_dot_ij, sum_j dS_ij (zero in exact arithmetic), and of
+    // their absolute sums, which only set the scale of a threshold and are sampled on every fourth key.
     float r4 = 0.f, r7 = 0.f, a4 = 0.f, a7 = 0.f;
 
     auto compute = [&](const elem_t* slot, int k0) {
@@ -187,13 +201,17 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                     const float dts = pj * (w[t][j] - s4);
                     w[t][j] = dts;
                     xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s7d));
-                    r4 += dts;
-                    if (j == 0) a4 += fabsf(dts);
+                    if constexpr (!SECOND) {
+                        r4 += dts;
+                        if (j == 0) a4 += fabsf(dts);
+                    }
                 } else {
                     xy[t][j] = pj * (xy[t][j] - s7d);
                 }
-                r7 += xy[t][j];
-                if (j == 0) a7 += fabsf(xy[t][j]);
+                if constexpr (!SECOND) {
+                    r7 += xy[t][j];
+                    if (j == 0) a7 += fabsf(xy[t][j]);
+                }
             }
         };
         // the second key tile's MFMA chains run under the first tile's element-wise arithmetic
@@ -202,6 +220,10 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         scores(1);
         pointwise(0);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MEASURE) {  // a launch that only measures the residues
+            pointwise(1);
+            return;
+        }
         // the transposed operands of the output contractions are read one step ahead, the first ones
         // under the second tile's element-wise arithmetic
         u32x4 ak = lds_a_tr16<HD>(sK, 0, lane), atk;
@@ -238,104 +260,24 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         if (i > 0 && issued < ns) issue_next();
         if (wave_active) compute(ring + (i % R) * SM::slot, i * kStageRows);
     }
-    // the residues of the row sums (see the top of the file); the four lanes of a query hold its keys
-    r4 = group_sum(r4);
-    r7 = group_sum(r7);
-    a4 = 4.0f * group_sum(a4);
-    a7 = 4.0f * group_sum(a7);
-    if (g == 0) {
-        p.s4[so] = s4 + r4;
-        p.s7d[so] = s7d + r7;
-    }
-    // A residue matters where it is not small against the rounding of the tiles it is spread over:
-    // |rho| against tau * sum_j |tile_ij|, tau = the spacing of the 16-bit format.  NaN compares false.
-    const bool wanted = qvalid && (fabsf(r4) > p.rowfix_tau * a4 || fabsf(r7) > p.rowfix_tau * a7);
-    const bool repair = p.rowfix == 2 || (p.rowfix == 1 && workgroup_barrier_or(wanted));
-    if (repair) {
-        // Second pass over the keys: P K into pk and (P*N) K + P K_dot into t2, with the 16-bit P and P*N
-        // as B operands (the terms they correct are themselves small).
-        workgroup_barrier();  // every wave is done with the ring of the first pass
-        using Plan2 = CopyPlan<HD, HAS_G ? 2 : 1, 1, kXThreads16>;
-        constexpr int SPT2 = Plan2::N;
-        Plan2 plan2;
-        if constexpr (HAS_G)
-            plan2.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl}, Src{p.tk.head(b, h), p.tk.sl});
-        else
-            plan2.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl});
-        int issued2 = 0;
-        auto issue2 = [&]() {
-            plan2.issue(ring + (issued2 % R) * SM::slot, p.Lk - issued2 * kStageRows);
-            ++issued2;
-        };
-        while (issued2 < R && issued2 < ns) issue2();
-        f32x4 pk[DT], t2[DT];
-#pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            pk[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            t2[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (!SECOND) {
+        // the residues of the row sums (see the top of the file); the four lanes of a query hold its keys
+        r4 = group_sum(r4);
+        r7 = group_sum(r7);
+        a4 = 4.0f * group_sum(a4);
+        a7 = 4.0f * group_sum(a7);
+        if (g == 0) {
+            p.s4[so] = s4 + r4;
+            p.s7d[so] = s7d + r7;
         }
-        auto compute2 = [&](const elem_t* slot, int k0) {
-            const elem_t* sK = slot;
-            const elem_t* sTK = slot + SE;
-            f32x4 s[2], ts[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-                ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int c = 0; c < KC; ++c) {
-                    const u32x4 ak = lds_a_rows16<HD>(sK, t, c, n, g);
-                    s[t] = T::mfma16(ak, qB[c], s[t]);
-                    if constexpr (HAS_G) {
-                        ts[t] = T::mfma16(ak, tqB[c], ts[t]);
-                        const u32x4 atk = lds_a_rows16<HD>(sTK, t, c, n, g);
-                        ts[t] = T::mfma16(atk, qB[c], ts[t]);
-                    }
-                }
-            }
-            const bool ragged = k0 + kStageRows > p.Lk;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float pj = fast_exp2(fmaf(s[t][j], sl2, -lse2));
-                    if (ragged && k0 + 16 * t + 4 * g + j >= p.Lk) pj = 0.f;
-                    s[t][j] = pj;
-                    if constexpr (HAS_G) ts[t][j] = pj * fmaf(ts[t][j], p.scale, -mu);
-                }
-            }
-            const u32x4 pB = pack_b16<T>(s[0], s[1]);
-            u32x4 pnB;
-            if constexpr (HAS_G) pnB = pack_b16<T>(ts[0], ts[1]);
-#pragma unroll
-            for (int d = 0; d < DT; ++d) {
-                const u32x4 ak = lds_a_tr16<HD>(sK, 16 * d, lane);
-                pk[d] = T::mfma16(ak, pB, pk[d]);
-                if constexpr (HAS_G) {
-                    t2[d] = T::mfma16(ak, pnB, t2[d]);
-                    const u32x4 atk = lds_a_tr16<HD>(sTK, 16 * d, lane);
-                    t2[d] = T::mfma16(atk, pB, t2[d]);
-                }
-            }
-        };
-        for (int i = 0; i < ns; ++i) {
-            wait_stages<SPT2>(issued2 - 1 - i);
-            workgroup_barrier();
-            if (i > 0 && issued2 < ns) issue2();
-            if (wave_active) compute2(ring + (i % R) * SM::slot, i * kStageRows);
+        // A residue matters where it is not small against the rounding of the tiles it is spread over:
+        // |rho| against tau * sum_j |tile_ij|, tau = the unit roundoff of the 16-bit format.  NaN compares false.
+        const bool wanted = qvalid && (fabsf(r4) > p.rowfix_tau * a4 || fabsf(r7) > p.rowfix_tau * a7);
+        if (p.rowfix == 1) {
+            const bool any = workgroup_barrier_or(wanted);
+            if (tid == 0) p.flags[bid] = any ? 1 : 0;
         }
-#pragma unroll
-        for (int d = 0; d < DT; ++d) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if constexpr (HAS_G) {
-                    dtq[d][j] = fmaf(-r4, pk[d][j], dtq[d][j]);
-                    dq[d][j] -= fmaf(r4, t2[d][j], r7 * pk[d][j]);
-                } else {
-                    dq[d][j] = fmaf(-r7, pk[d][j], dq[d][j]);
-                }
-            }
-        }
+        if constexpr (MEASURE) return;  // the second launch writes dQ, dQ_dot
     }
     workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
     if (!wave_active) return;

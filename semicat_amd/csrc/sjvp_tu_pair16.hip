@@ -15,9 +15,18 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     // the column-owned one; workgroups of four waves own 64 positions
     constexpr int XR = HD == 128 ? 2 : 3;  // ring depth
     int rc = SJVP_OK;
-    if (parts & SJVP_BWD_ROW)
-        rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, (HD == 128 ? 2 : 3)>,
-                    BH * (p.Lr / kXOwned16), Row16Smem<HD, XR, HAS_G>::bytes, stream, p, kXThreads16);
+    if (parts & SJVP_BWD_ROW) {
+        constexpr int OCC = HD == 128 ? 2 : 3;
+        const int grid = BH * (p.Lr / kXOwned16);
+        constexpr int smem = Row16Smem<HD, XR, HAS_G>::bytes;
+        // "always": a launch that measures the row-sum residues, then one that computes with the corrected
+        // sums; otherwise the pass itself and, unless switched off, a second launch in which the workgroups
+        // whose residues call for it run again
+        if (p.rowfix == 2) rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 1>, grid, smem, stream, p, kXThreads16);
+        else rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 0>, grid, smem, stream, p, kXThreads16);
+        if (rc == SJVP_OK && p.rowfix != 0)
+            rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 2>, grid, smem, stream, p, kXThreads16);
+    }
     if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
     const int grid = BH * ((p.Lk + kXOwned16 - 1) / kXOwned16);
     using CS = Col16Smem<HD, XR, HAS_DO, HAS_G>;

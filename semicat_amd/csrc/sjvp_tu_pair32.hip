@@ -9,9 +9,16 @@ namespace {
 template <typename T, int HD, bool HAS_DO, bool HAS_G>
 int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     int rc = SJVP_OK;
-    if (parts & SJVP_BWD_ROW)
-        rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G>, BH * p.q_blocks, RowSmem<HD, HAS_G>::bytes, stream, p,
-                    kThreads);
+    if (parts & SJVP_BWD_ROW) {
+        const int grid = BH * p.q_blocks;
+        constexpr int smem = RowSmem<HD, HAS_G>::bytes;
+        // "always": measure the row-sum residues, then compute with the corrected sums; otherwise the pass
+        // and, unless switched off, a second launch for the workgroups whose residues call for it
+        if (p.rowfix == 2) rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G, false, 1>, grid, smem, stream, p, kThreads);
+        else rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G, false, 0>, grid, smem, stream, p, kThreads);
+        if (rc == SJVP_OK && p.rowfix != 0)
+            rc = launch(bwd_row_kernel<T, HD, HAS_DO, HAS_G, false, 2>, grid, smem, stream, p, kThreads);
+    }
     if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
     const int col_grid = BH * p.k_blocks;
     using SM = ColSmem<HD, HAS_DO, HAS_G>;

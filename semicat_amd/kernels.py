@@ -81,8 +81,9 @@ _REPAIR_MODES = {"off": _lib.SJVP_REPAIR_OFF, "auto": _lib.SJVP_REPAIR_AUTO, "al
 def set_row_sum_repair(mode: str) -> str:
     """How the backward deals with what the rounding of ``o``, ``to`` leaves in its row sums (the
     reference forms those sums from the probabilities, flash_jvp_backward.py:2012-2290): ``"off"``,
-    ``"auto"`` (default: a second pass over the keys for the workgroups whose rows need it) or
-    ``"always"`` (everywhere, and the row + column launches also where the single launch would run).
+    ``"auto"`` (default: a second launch of the row-owned kernel recomputes dq, dq_dot with the corrected
+    sums for the workgroups whose rows need it) or ``"always"`` (for every row, and the row + column
+    launches also where the single launch would run).
     Process-wide; returns the previous mode."""
     if mode not in _REPAIR_MODES:
         raise ValueError(f"row-sum repair mode must be one of {sorted(_REPAIR_MODES)}, got {mode!r}")

@@ -224,9 +224,9 @@ def test_row_sums_from_rounded_outputs_leave_a_coherent_residue():
 
 
 def test_repaired_row_sums_match_the_sums_from_the_probabilities():
-    """The repaired form of the row-sum model (residues of dS_dot, dS summed over the keys, corrected
-    sums for the key side, P K and (P*N) K + P K_dot terms for the query side) is as accurate as the
-    reference's form on the cases where the sums of the rounded outputs alone fail: the 255-key case,
+    """The repaired form of the row-sum model (residues of dS_dot, dS summed over the keys and added to
+    the sums, every gradient formed again with the corrected sums) is as accurate as the reference's
+    form on the cases where the sums of the rounded outputs alone fail: the 255-key case,
     a saturated single row in fp16 (0.9998 of the probability on one of five keys: 0.5-0.6 relative
     error without the repair) and constructed saturated rows in bf16."""
     cases = []

@@ -874,8 +874,8 @@ def test_row_sum_residues_are_repaired_on_the_row_and_column_pair(K):
     probabilities as the reference's preprocess kernel does (flash_jvp_backward.py:2266-2287).  On rows
     where sum_j P (W - s4) cancels strongly (two query rows, 255 keys, logits of scale 2) that form
     alone leaves 1.4e-2 on dq_dot, dk_dot.  The row-owned launch measures the residue, hands the
-    column-owned launch corrected sums and repairs its own dq, dq_dot with a second pass: every output
-    keeps the plain gate."""
+    column-owned launch corrected sums, and its second launch recomputes dq, dq_dot with them: every
+    output keeps the plain gate."""
     x = orc.make_inputs(2, 1, 2, 255, 40, seed=1062, primal_scale=2.0, tangent_scale=0.3, dtype=torch.bfloat16)
     err, models = _row_sum_report(x, run_hip(K, x), torch.bfloat16)
     assert models["sums from O, TO"]["dtq"] > TOL_16BIT  # the case does exercise the residue
@@ -912,11 +912,37 @@ def test_saturated_rows_on_the_row_and_column_pair(K, dtype, D, Lk, only_dto):
         assert e <= TOL_16BIT, (n, e)
 
 
+@pytest.mark.parametrize("D,Lk,dtype,mode", [(80, 133, torch.float16, "auto"), (36, 70, torch.bfloat16, "auto"),
+                                             (128, 133, torch.bfloat16, "always"), (64, 100, torch.bfloat16, "auto")])
+def test_saturated_rows_on_the_register_staged_pair(K, repair_mode, D, Lk, dtype, mode):
+    """The same repair in the 32-wide register-staged kernels (base pointers off the 16-byte grid, or a
+    head dimension that is not a multiple of 8): saturated rows, up to 0.999998 of the probability on one
+    key, keep the gate for every output."""
+    repair_mode(mode)
+    x = orc.make_inputs(1, 2, 3, Lk, D, seed=5, primal_scale=1.0, tangent_scale=0.3, dtype=dtype)
+    for i in range(3):
+        x["k"][:, :, 7 + 20 * i, :] = (x["q"][:, :, i, :].float() * 1.5).to(dtype)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    d = {}
+    for n, t in x.items():
+        buf = torch.zeros(t.numel() + 1, dtype=t.dtype, device="cuda")
+        d[n] = buf[1:].view(t.shape).copy_(t.cuda())
+    o, to, lse, mu, _ = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g)}}
+    model = orc.row_sum_rounding_model(*[x[n] for n in orc.TENSOR_ORDER], dtype=dtype)
+    worst = max(orc.rel_frobenius(torch.from_numpy(model[n]), ref[n]) for n in ("dtq", "dtk"))
+    assert worst > TOL_16BIT, worst  # unrepaired, the case fails the gate
+    assert_parity(res, ref, TOL_16BIT, label=f"saturated rows, register-staged pair D={D} Lk={Lk}")
+
+
 def test_row_sum_repair_modes(K, repair_mode):
     """sjvp_set_row_sum_repair: "off" still hands the column-owned launch the corrected sums (dk, dk_dot
     keep the gate on the 255-key case, dq_dot carries the residue); "always" takes the row + column pair
-    with the repair also where the single launch would run (100 keys), and is reference-grade there,
-    while the single launch stays within 1.5x of what the row-sum model predicts for its form."""
+    (a measuring launch, then every row computed with the corrected sums) also where the single launch
+    would run (100 keys), and is reference-grade there, while the single launch stays within 1.5x of what
+    the row-sum model predicts for its form."""
     x = orc.make_inputs(2, 1, 2, 255, 40, seed=1062, primal_scale=2.0, tangent_scale=0.3, dtype=torch.bfloat16)
     repair_mode("off")
     err, models = _row_sum_report(x, run_hip(K, x), torch.bfloat16)
