@@ -213,8 +213,9 @@ def test_library_exports_every_declared_symbol(repo_root):
         assert hasattr(lib, name), name
     L = _lib.load()
     assert L.sjvp_version() == int(re.search(r"#define SJVP_VERSION (\d+)", header).group(1))
-    assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4
-    assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4
+    # 12 bytes per statistic row (rows rounded up to 128 per head) + one 4-byte flag per 64 rows
+    assert L.sjvp_bwd_workspace_bytes(64, 12, 128, 128, 64, 0) == 3 * 64 * 12 * 128 * 4 + 64 * 12 * 2 * 4
+    assert L.sjvp_bwd_workspace_bytes(1, 1, 129, 7, 64, 0) == 3 * 256 * 4 + 4 * 4
     for code in range(0, -12, -1):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
