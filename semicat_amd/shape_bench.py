@@ -1,5 +1,5 @@
 """Step time of the attention-JVP forward + backward at any shape:
-``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16|fp32io|fp32cast|fp32lib] [--steps K]``.
+``python -m semicat_amd.shape_bench --shape B H L D [--keys Lk] [--dtype bf16|fp16|fp32|fp32io|fp32cast|fp32lib] [--steps K]``.
 
 The same measurement as the headline benchmark (planned launches through the C ABI on one stream,
 0.3 s of untimed load first, then K timed steps; random q, k, v ~ 0.5 N(0,1), tangents ~ 0.1 N(0,1),
@@ -7,6 +7,7 @@ cotangents ~ N(0,1)), for the shapes the headline benchmark does not cover: long
 head dimensions, keys and queries of different lengths.  Work model 42*B*H*Lq*Lk*D flop per step.
 Prints one JSON line.  A companion measurement, not the headline figure.
 
+``--dtype fp32`` times the library's fp32 correctness mode (fp32 arithmetic on the vector ALUs);
 ``--dtype fp32io`` and ``fp32cast`` time the two ways of serving a float32 caller with bf16 arithmetic
 (the dtype policy of semicat/jvp_utils/functional.py:318-332): the casts folded into the kernels
 (float32 tensors handed over as they are, SJVP_FP32_BF16), or torch casts around the 16-bit kernels
@@ -29,7 +30,7 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--shape", type=int, nargs=4, metavar=("B", "H", "L", "D"), default=(128, 12, 256, 64))
     ap.add_argument("--keys", type=int, default=None, help="key/value length (default: L)")
-    ap.add_argument("--dtype", choices=("bf16", "fp16", "fp32io", "fp32cast", "fp32lib"), default="bf16")
+    ap.add_argument("--dtype", choices=("bf16", "fp16", "fp32", "fp32io", "fp32cast", "fp32lib"), default="bf16")
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     a = ap.parse_args(argv)
@@ -43,7 +44,7 @@ def main(argv=None) -> int:
     Lk = a.keys or Lq
     fp32 = a.dtype.startswith("fp32")
     dt = torch.float32 if fp32 else (torch.bfloat16 if a.dtype == "bf16" else torch.float16)
-    code = _lib.SJVP_FP32_BF16 if a.dtype == "fp32io" else (_lib.SJVP_FP16 if a.dtype == "fp16" else _lib.SJVP_BF16)
+    code = {"fp32io": _lib.SJVP_FP32_BF16, "fp32": _lib.SJVP_FP32, "fp16": _lib.SJVP_FP16}.get(a.dtype, _lib.SJVP_BF16)
     g = torch.Generator(device=dev).manual_seed(0)
 
     def rnd(L, s):
@@ -139,7 +140,8 @@ def main(argv=None) -> int:
     unit = float(B) * H * Lq * Lk * D
     print(json.dumps({
         "workload": f"attention JVP fwd+bwd, B={B} H={H} Lq={Lq} Lk={Lk} D={D}, "
-                    + {"fp32io": "fp32 tensors, casts folded into the kernels, bf16 arithmetic",
+                    + {"fp32": "fp32 tensors and fp32 arithmetic on the vector ALUs (the correctness mode)",
+                       "fp32io": "fp32 tensors, casts folded into the kernels, bf16 arithmetic",
                        "fp32lib": "fp32 tensors, the library's cast launches around the bf16 kernels",
                        "fp32cast": "fp32 tensors, torch casts around the bf16 kernels"}.get(
                            a.dtype, f"{a.dtype} in / fp32 acc") + ", both cotangents",

@@ -96,3 +96,20 @@ def model_step(net: nn.Module, x1: Tensor, in_shape: tuple[int, ...], sd_prop: f
     if split == 0:
         return vf, None
     return vf, lag_self_distillation_loss(net, x0[:split], x1[:split])
+
+
+def compile_network(net: torch.nn.Module, backend: str = "aot_eager", **kwargs):
+    """``torch.compile(net, backend=...)`` as the reference wraps its network (semicat.py:340-345), with
+    the one backend that is known to fail here refused up front: on an MI355X box the reference's default,
+    ``backend="inductor"``, once ended in a segmentation fault of the Python process while it compiled the
+    PyTorch layers around the op (torch 2.10.0+rocm7.0, triton 3.6.0; cause not identified, not run
+    again), so a network on a GPU is compiled with ``"aot_eager"`` (tested: both losses and the gradients
+    equal the unwrapped network's) or left in eager mode.  On the CPU, inductor compiles the same
+    network and matches eager.  The op itself is a graph break under every backend
+    (``torch._dynamo.disable``, as functional.py:272)."""
+    on_gpu = any(p.is_cuda for p in net.parameters())
+    if backend == "inductor" and on_gpu:
+        raise RuntimeError("backend='inductor' around a network on the GPU is not supported by this build: a run "
+                           "on an MI355X box ended in a segmentation fault while inductor compiled the layers "
+                           "around the op; use backend='aot_eager' or eager mode")
+    return torch.compile(net, backend=backend, **kwargs)

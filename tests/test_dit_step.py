@@ -281,3 +281,33 @@ def test_network_under_torch_compile_gpu():
     vf1, sd1, g1 = run(torch.compile(net, backend="aot_eager"))
     assert abs(vf1 - vf0) <= 1e-5 * abs(vf0) and abs(sd1 - sd0) <= 1e-5 * abs(sd0)
     assert (g1 - g0).norm() <= 1e-5 * g0.norm()
+
+
+def test_compile_network_refuses_inductor_on_a_gpu_and_passes_other_backends_through():
+    """The helper that wraps the network as the reference does: "aot_eager" (and anything on the CPU) goes
+    to torch.compile, inductor for a network on a GPU raises before anything is compiled."""
+    from semicat_amd.train_step import compile_network
+    net = torch.nn.Linear(4, 4)
+    compiled = compile_network(net, backend="aot_eager")
+    x = torch.randn(2, 4)
+    assert torch.allclose(compiled(x), net(x))
+
+    class OnGpu(torch.nn.Module):  # stands for a network whose parameters live on a GPU
+        def parameters(self, recurse=True):
+            class P:
+                is_cuda = True
+            return iter([P()])
+
+    with pytest.raises(RuntimeError, match="inductor"):
+        compile_network(OnGpu(), backend="inductor")
+
+
+@pytest.mark.gpu
+@pytest.mark.skip(reason="torch.compile(net, backend='inductor') on an MI355X box ended in a segmentation fault of "
+                         "the Python process while inductor compiled the PyTorch layers around the op (torch "
+                         "2.10.0+rocm7.0, triton 3.6.0); no cause has been shown, so the case stays off the GPU. "
+                         "On the CPU inductor compiles the network and matches eager, and triton 3.6.0 "
+                         "cross-compiles a kernel for gfx950 without a GPU.")
+def test_network_under_inductor_gpu():
+    from semicat_amd.train_step import compile_network  # noqa: F401
+    raise AssertionError("not run: see the skip reason")
