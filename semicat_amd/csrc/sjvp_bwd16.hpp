@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     auto issue_next = [&]() {
         elem_t* slot = ring + (issued % R) * SM::slot;
         const int row0 = issued * kStageRows;
-        plan.issue(slot, p.Lq - row0);
+        plan.issue(slot, p.Lq - row0, p.D == HD && row0 + kStageRows <= p.Lq);
         // raw lse (wave 0) and mu (wave 1) of the stage's rows (rows < Lr exist); every wave issues
         // exactly one 4-byte LDS-DMA instruction, the others as a placeholder into the sink
         float* raw = reinterpret_cast<float*>(slot + oST);
@@ -166,8 +166,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             float* fin = raw + 2 * kStageRows;
             fin[0 * kStageRows + r] = raw[r] * kLog2e;
             fin[1 * kStageRows + r] = HAS_G ? raw[kStageRows + r] : 0.f;
-            fin[2 * kStageRows + r] = s4;
-            fin[3 * kStageRows + r] = s7d;
+            fin[2 * kStageRows + r] = -s4;  // the W and XY tiles start from these instead of subtracting them
+            fin[3 * kStageRows + r] = -s7d;
         }
     };
 
@@ -192,8 +192,10 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         auto scores = [&](int t) __attribute__((always_inline)) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            // W - s4 and XY - s7d: the accumulators start at the negated row sums (register j of tile t is
+            // query 16t + 4g + j)
+            w[t] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + 16 * t + 4 * g);
+            xy[t] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + 16 * t + 4 * g);
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
                 const u32x4 aq = lds_a_rows16<HD>(sQ, t, c, n, g);
@@ -213,27 +215,30 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             }
         };
         // in place: s -> P, ts -> P_dot, w -> dS_dot, xy -> dS  (register j of tile t is query 16t + 4g + j)
-        auto pointwise = [&](int t) __attribute__((always_inline)) {
+        auto pointwise_of = [&](int t, auto ragged_tag) __attribute__((always_inline)) {
             const int r0 = 16 * t + 4 * g;
             const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
             const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
-            const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
-            const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 float pj = fast_exp2(fmaf(s[t][j], sl2, -lse4[j]));
-                if (ragged_keys && key_padded) pj = 0.f;
+                if (decltype(ragged_tag)::value && key_padded) pj = 0.f;
                 s[t][j] = pj;
                 if constexpr (HAS_G) {
                     const float nn = fmaf(ts[t][j], p.scale, -mu4[j]);
-                    const float dts = pj * (w[t][j] - s44[j]);
+                    const float dts = pj * w[t][j];
                     w[t][j] = dts;
-                    xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[j]));
+                    xy[t][j] = fmaf(dts, nn, pj * xy[t][j]);
                     ts[t][j] = pj * nn;
                 } else {
-                    xy[t][j] = pj * (xy[t][j] - s74[j]);
+                    xy[t][j] = pj * xy[t][j];
                 }
             }
+        };
+        // a wave whose sixteen keys all exist (wave-uniform) skips the selects of the padded keys
+        auto pointwise = [&](int t) __attribute__((always_inline)) {
+            if (ragged_keys) pointwise_of(t, std::true_type{});
+            else pointwise_of(t, std::false_type{});
         };
         // the second tile's MFMA chains run under the first tile's pointwise arithmetic
         scores(0);

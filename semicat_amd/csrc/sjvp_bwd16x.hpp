@@ -104,7 +104,8 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     const int ns = (p.Lk + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
-        plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows);
+        plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows,
+                   p.D == HD && (issued + 1) * kStageRows <= p.Lk);
         ++issued;
     };
     while (issued < R && issued < ns) issue_next();
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     auto issue_next = [&]() {
         elem_t* slot = ring + (issued % R) * SM::slot;
         const int row0 = issued * kStageRows;
-        plan.issue(slot, p.Lq - row0);
+        plan.issue(slot, p.Lq - row0, p.D == HD && row0 + kStageRows <= p.Lq);
         // the four statistic arrays (lse2, mu, s4, s7d) of the stage's rows, one per wave, 32 lanes
         // each (rows < Lr exist in all of them); every wave issues exactly one 4-byte LDS-DMA
         const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;
@@ -604,7 +605,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
     auto issue_next = [&]() {
         elem_t* slot = ring + (issued % R) * SM::slot;
         const int row0 = issued * kStageRows;
-        plan.issue(slot, p.Lq - row0);
+        plan.issue(slot, p.Lq - row0, p.D == HD && row0 + kStageRows <= p.Lq);
         // the four statistic arrays of the stage's rows by waves 0..3; the others issue a placeholder
         if (wave < 4) {
             const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;

@@ -83,7 +83,8 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
     const int ns = (p.Lk + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
-        plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows);
+        plan.issue(ring + (issued % R) * SM::slot, p.Lk - issued * kStageRows,
+                   p.D == HD && (issued + 1) * kStageRows <= p.Lk);
         ++issued;
     };
     while (issued < (SPB == 2 ? 2 : R) && issued < ns) issue_next();

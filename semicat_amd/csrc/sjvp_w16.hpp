@@ -99,8 +99,19 @@ struct CopyPlan {
     }
 
     // Copy the next window into `region`; rows_left = rows of the window that exist (zero fill beyond).
-    __device__ __forceinline__ void issue(elem_t* region, int rows_left) {
+    // `whole` (wave-uniform): the caller knows that every row of the window exists and that D covers every
+    // chunk, so every lane copies and nothing is predicated (a few instructions per copy instead of the
+    // forty of the general form, which matters in loops that are bound by instruction issue).
+    __device__ __forceinline__ void issue(elem_t* region, int rows_left, bool whole = false) {
         const uint32_t base = lds_addr(region);
+        if (total % NT == 0 && whole) {
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                dma16(src[i], base + wbase[i]);
+                src[i] += adv[i];
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             bool valid = false;
