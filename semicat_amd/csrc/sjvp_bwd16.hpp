@@ -98,7 +98,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         else
             own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
                           Src{p.v.head(b, h), p.v.sl});
-        own_plan.issue(ownK, p.Lk);
+        own_plan.issue(ownK, p.Lk, p.D == HD && p.Lk == kOwned16);
     }
     using StagePlan = CopyPlan<HD, SM::nt, 1>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(kThreads16, OCC) void fwd16_kernel(const FwdParams 
                           Src{p.tq.head(b, h), p.tq.sl});
         else
             own_plan.init(tid, q0, p.D, smem_raw + SM::sink, Src{p.q.head(b, h), p.q.sl});
-        own_plan.issue(own, p.Lq - q0);
+        own_plan.issue(own, p.Lq - q0, p.D == HD && q0 + kOwned16 <= p.Lq);
     }
     using StagePlan = CopyPlan<HD, SM::nt, 1>;
     constexpr int SPT = StagePlan::N;

@@ -59,42 +59,69 @@ struct CopyPlan {
     uint32_t sink;
 
     // Tensors are passed one by one (not as an array) so that the wave-uniform choice among them
-    // stays a chain of scalar selects.
+    // stays a chain of scalar selects.  NT and the chunks of a slab are powers of two, so a thread's
+    // positions are the SAME chunk (row within the slab, column) of successive slabs (NT >= chunks) or
+    // of successive parts of one slab (NT < chunks): the column and the swizzle are computed once and
+    // the slab index is a scalar, which keeps this set-up to a few instructions per position (it runs
+    // once per workgroup, and a workgroup with a short loop lives only some ten thousand cycles).
     __device__ __forceinline__ void init(int tid, int first_row, int D, const void* sink_lds, Src t0,
                                          Src t1 = Src{nullptr, 0}, Src t2 = Src{nullptr, 0},
                                          Src t3 = Src{nullptr, 0}, Src t4 = Src{nullptr, 0},
                                          Src t5 = Src{nullptr, 0}) {
         static_assert(NTENS <= 6, "at most six tensors per copy");
+        static_assert(NT % chunks == 0 || chunks % NT == 0, "thread count and slab size are powers of two");
         constexpr int CH = HD / 8;
         any = t0.ptr;
         sink = lds_addr(sink_lds);
+        const int q0 = tid % chunks;                      // position within its slab for i = 0
+        const int c8 = 8 * ((q0 % CH) ^ swz<HD>(q0 / CH));  // rows r and r + 16 k share their swizzle
+        static_assert(NT >= chunks || (NT / CH) % 16 == 0, "parts of a slab start at multiples of 16 rows");
+        const int j0 = __builtin_amdgcn_readfirstlane(tid / chunks);  // slab of position i = 0 (wave-uniform)
+        const bool col_ok = c8 < D;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
-            const int p = tid + i * NT;
-            on[i] = p < total;
-            const int j = p / chunks, q = p % chunks;
-            const int r = q / CH;
-            const int c8 = 8 * ((q % CH) ^ swz<HD>(r));
-            const int tensor = __builtin_amdgcn_readfirstlane(j / SPTN);
-            const elem_t* ptr = t0.ptr;
-            int64_t sl = t0.sl;
-            auto pick = [&](int k, const Src& t) {
-                if (k < NTENS && tensor == k) {
-                    ptr = t.ptr;
-                    sl = t.sl;
+            int j, r;
+            if constexpr (NT >= chunks) {
+                j = j0 + (NT / chunks) * i;
+                r = q0 / CH;
+            } else {
+                j = i / (chunks / NT);
+                r = q0 / CH + (NT / CH) * (i % (chunks / NT));
+            }
+            on[i] = j < NS;
+            // the tensor of slab j: known at compile time where a thread's slabs never straddle two tensors,
+            // else one of NT / chunks neighbours, chosen by the (wave-uniform) slab of position 0
+            const Src ts[6] = {t0, t1, t2, t3, t4, t5};
+            const elem_t* ptr;
+            int64_t sl;
+            if constexpr (NT < chunks) {
+                constexpr int PPS = chunks / NT;
+                ptr = ts[(i / PPS) / SPTN < NTENS ? (i / PPS) / SPTN : 0].ptr;
+                sl = ts[(i / PPS) / SPTN < NTENS ? (i / PPS) / SPTN : 0].sl;
+            } else if constexpr (SPTN % (NT / chunks) == 0) {
+                constexpr int SPI = NT / chunks;
+                ptr = ts[(SPI * i) / SPTN < NTENS ? (SPI * i) / SPTN : 0].ptr;
+                sl = ts[(SPI * i) / SPTN < NTENS ? (SPI * i) / SPTN : 0].sl;
+            } else {
+                static_assert(NT < chunks || SPTN % (NT / chunks) == 0 || SPTN == 1, "slabs per tensor");
+                constexpr int SPI = NT / chunks;
+                ptr = ts[SPI * i < NTENS ? SPI * i : 0].ptr;
+                sl = ts[SPI * i < NTENS ? SPI * i : 0].sl;
+#pragma unroll
+                for (int k = 1; k < SPI; ++k) {
+                    if (SPI * i + k < NTENS && j0 == k) {
+                        ptr = ts[SPI * i + k < NTENS ? SPI * i + k : 0].ptr;
+                        sl = ts[SPI * i + k < NTENS ? SPI * i + k : 0].sl;
+                    }
                 }
-            };
-            pick(1, t1);
-            pick(2, t2);
-            pick(3, t3);
-            pick(4, t4);
-            pick(5, t5);
-            row[i] = 32 * (j % SPTN) + r;
-            src[i] = ptr + (int64_t)(first_row + row[i]) * sl + c8;
+            }
+            const int slab_row = 32 * (j % SPTN);  // scalar
+            row[i] = slab_row + r;
+            src[i] = (ptr + (int64_t)(first_row + slab_row) * sl) + ((int64_t)r * sl + c8);
             adv[i] = 32 * SPTN * sl;
-            ok[i] = c8 < D;
-            wbase[i] = (uint32_t)((p & ~63) * 16);
-            pos[i] = (uint32_t)(p * 16);
+            ok[i] = col_ok;
+            wbase[i] = (uint32_t)(((tid & ~63) + i * NT) * 16);
+            pos[i] = (uint32_t)((tid + i * NT) * 16);
         }
     }
 
