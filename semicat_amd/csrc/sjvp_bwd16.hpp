@@ -24,7 +24,8 @@ namespace sjvp {
 // read into registers the same memory is the bounce tile dS (, dS_dot): [128 keys][32 queries + pad]]
 // [ring of query stages: Q | [Q_dot | G] | [dO] | O | [TO] | raw lse, mu | lse2, mu, s4, s7d]
 // [staging tile of a stage's dQ (, dQ_dot)][sink]
-// After the last stage the ring doubles as the per-wave staging tiles of the output stores.
+// In the last stage the two ring slots that no stage uses again hold the per-wave staging tiles of the
+// output stores.
 template <int HD, int R, bool HAS_DO, bool HAS_G>
 struct Fused16Smem {
     static constexpr int nt = 2 + (HAS_G ? 3 : 0) + (HAS_DO ? 1 : 0);
@@ -41,7 +42,6 @@ struct Fused16Smem {
     static constexpr int qstage = (HAS_G ? 2 : 1) * kStageRows * qpitch;
     static constexpr int sink = (own_k + vregion + R * slot + qstage) * (int)sizeof(elem_t);
     static constexpr int bytes = sink + kSink16;
-    static_assert(R * slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
 // ROPE: q, k and their tangents are rotated by p.rope once they are in LDS (own K, K_dot rows in the
@@ -88,18 +88,6 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     const bool ragged_keys = wave * 16 + 16 > p.Lk;
     const bool key_padded = wave * 16 + n >= p.Lk;
 
-    // own rows first (they land first), then the ring
-    {
-        CopyPlan<HD, HAS_G ? 16 : 8, 4> own_plan;
-        if constexpr (HAS_G)
-            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
-                          Src{p.tk.head(b, h), p.tk.sl}, Src{p.v.head(b, h), p.v.sl},
-                          Src{p.tv.head(b, h), p.tv.sl});
-        else
-            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
-                          Src{p.v.head(b, h), p.v.sl});
-        own_plan.issue(ownK, p.Lk, p.D == HD && p.Lk == kOwned16);
-    }
     using StagePlan = CopyPlan<HD, SM::nt, 1>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
     StagePlan plan;
@@ -133,6 +121,20 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         ++issued;
     };
     issue_next();
+    // The first stage is issued before the own rows: it lands first and its row sums are formed while the
+    // own rows (four times its size) are still on their way.
+    constexpr int OWN = (HAS_G ? 16 : 8) * Slab<HD>::chunks / kThreads16;  // own-row copies per wave
+    {
+        CopyPlan<HD, HAS_G ? 16 : 8, 4> own_plan;
+        if constexpr (HAS_G)
+            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
+                          Src{p.tk.head(b, h), p.tk.sl}, Src{p.v.head(b, h), p.v.sl},
+                          Src{p.tv.head(b, h), p.tv.sl});
+        else
+            own_plan.init(tid, 0, p.D, smem_raw + SM::sink, Src{p.k.head(b, h), p.k.sl},
+                          Src{p.v.head(b, h), p.v.sl});
+        own_plan.issue(ownK, p.Lk, p.D == HD && p.Lk == kOwned16);
+    }
     const float sl2 = p.scale * kLog2e;
 
     // Row sums of a landed stage: thread t < 256 handles row t/8, columns 8*(t%8) .. +7; the eight
@@ -373,8 +375,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
     };
 
-    // Only the own rows and stage 0 are waited for here; the later stages are issued once these
+    // Only stage 0 and the own rows are waited for here; the later stages are issued once these
     // have landed, so that their copies run under the arithmetic instead of ahead of it.
+    wait_stages<OWN>(1);  // everything but the OWN youngest copies of this wave: stage 0
+    workgroup_barrier();
+    row_sums(ring);
     wait_stages<SPT>(0);
     workgroup_barrier();
     if (issued < ns) issue_next();
@@ -406,8 +411,18 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             read_b_operands16<HD>(tvB, ownV + (4 + sidx) * SE, r, g);
         }
     }
-    row_sums(ring);
     rotate_stage(ring, 0);
+    // dK, dV (, dK_dot, dV_dot) of this wave's sixteen keys through its staging tile
+    auto key_gradients = [&](elem_t* stage_tile) {
+        const int row0 = wave * 16;
+        store_tile16<T, HD, ROPE>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane, &p.rope);
+        if constexpr (HAS_G)
+            store_tile16<T, HD, ROPE>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane,
+                                      &p.rope);
+        store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
+        if constexpr (HAS_G)
+            store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
+    };
     for (int i = 0; i < ns; ++i) {
         // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
         // every wave has read V, V_dot, whose memory the bounce tile takes over)
@@ -416,6 +431,15 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if (issued < ns && issued < i + R) issue_next();  // into the slot of stage issued - R <= i - 1
         elem_t* slot = ring + (i % R) * SM::slot;
         if (wave_active) tile(slot);
+        if (!ROPE && i == ns - 1 && wave_active) {
+            // The gradients of this wave's keys are complete.  They leave now, while step 3 of the last stage
+            // is still to come, through per-wave staging tiles in the two ring slots that no stage uses again
+            // (waves 0..3 in one, 4..7 in the other): the stores drain under the remaining arithmetic
+            // instead of after it.  (With the folded rotation the stores need registers that the stage loop
+            // cannot spare; they follow the loop there.)
+            static_assert(R >= 3 && SM::slot >= 4 * StoreStage16<HD>::elems, "two spare slots hold the staging tiles");
+            key_gradients(ring + ((i + 1 + (wave >> 2)) % R) * SM::slot + (wave & 3) * StoreStage16<HD>::elems);
+        }
         if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
         workgroup_barrier();
         if (i + 1 < ns) {
@@ -425,18 +449,12 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
         else row_outputs(i * kStageRows, std::false_type{});
     }
-    workgroup_barrier();  // every wave is done reading the ring: it becomes the store staging area
+    workgroup_barrier();  // the last stage's dQ (, dQ_dot) tiles are in their staging tile; the ring is free
     flush_rows((ns - 1) * kStageRows);
-    if (!wave_active) return;
-    elem_t* stage_tile = ring + wave * StoreStage16<HD>::elems;
-    const int row0 = wave * 16;
-    store_tile16<T, HD, ROPE>(stage_tile, p.dk.head(b, h), p.dk.sl, row0, p.Lk, p.D, dk, p.scale, lane, &p.rope);
-    if constexpr (HAS_G)
-        store_tile16<T, HD, ROPE>(stage_tile, p.dtk.head(b, h), p.dtk.sl, row0, p.Lk, p.D, dtk, p.scale, lane,
-                                  &p.rope);
-    store_tile16<T, HD>(stage_tile, p.dv.head(b, h), p.dv.sl, row0, p.Lk, p.D, dv, 1.0f, lane);
-    if constexpr (HAS_G)
-        store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
+    if constexpr (ROPE) {
+        static_assert(R * SM::slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
+        if (wave_active) key_gradients(ring + wave * StoreStage16<HD>::elems);
+    }
 }
 
 }  // namespace sjvp
