@@ -33,16 +33,24 @@ struct Fused16Smem {
     static constexpr int slot = nt * Slab<HD>::elems + stat_elems;
     static constexpr int own_k = (HAS_G ? 2 : 1) * 4 * Slab<HD>::elems;  // K (, K_dot)
     static constexpr int own_v = own_k;                                  // V (, V_dot)
-    static constexpr int bpitch = 48;  // elements per key row: 4 rows of a transposing read hit distinct banks
-    static constexpr int bounce_one = kOwned16 * bpitch;
-    static constexpr int bounce = (HAS_G ? 2 : 1) * bounce_one;
+    // bounce tile [128 keys][32 queries], 64 bytes per key: eight units of four queries, unit u of key y at
+    // position u ^ bounce_swz(y).  Two buffers (even and odd stages) of one tile per kind (dS, dS_dot).
+    static constexpr int bounce_one = kOwned16 * kStageRows;
+    static constexpr int bounce = 2 * (HAS_G ? 2 : 1) * bounce_one;
     static constexpr int vregion = own_v > bounce ? own_v : bounce;
-    // staging of a stage's dQ (, dQ_dot) tiles, [32 queries][HD + 8], so that they leave as whole rows
+    // staging of a stage's dQ (, dQ_dot) tiles, [32 queries][HD + 8], so that they leave as whole rows;
+    // two buffers (even and odd stages)
     static constexpr int qpitch = HD + 8;
-    static constexpr int qstage = (HAS_G ? 2 : 1) * kStageRows * qpitch;
+    static constexpr int qstage_one = (HAS_G ? 2 : 1) * kStageRows * qpitch;
+    static constexpr int qstage = 2 * qstage_one;
     static constexpr int sink = (own_k + vregion + R * slot + qstage) * (int)sizeof(elem_t);
     static constexpr int bytes = sink + kSink16;
 };
+
+// Position of unit u (four queries, 8 bytes) of key y in its 64-byte row of a bounce tile: with it the
+// 8-byte writes of a wave (16 keys x 4 units per instruction) and the transposing reads (4 keys x 4 units
+// per group of 16 lanes, groups 4 keys apart) spread over all banks.
+__device__ __forceinline__ int bounce_swz(int key) { return 4 * ((key >> 2) & 1) + 2 * ((key >> 3) & 1); }
 
 // ROPE: q, k and their tangents are rotated by p.rope once they are in LDS (own K, K_dot rows in the
 // prologue, each stage's Q, Q_dot slabs by the threads that do not form row sums), and the gradients
@@ -56,19 +64,20 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     constexpr int SE = Slab<HD>::elems;
     elem_t* ownK = reinterpret_cast<elem_t*>(smem_raw);  // K slabs 0..3, then K_dot slabs 0..3
     elem_t* ownV = ownK + SM::own_k;                      // V slabs 0..3, then V_dot slabs 0..3
-    elem_t* bounceS = ownV;                               // aliases V, V_dot after the prologue
-    elem_t* bounceT = ownV + SM::bounce_one;
+    elem_t* bounce0 = ownV;  // aliases V, V_dot after the prologue: [buffer][dS | dS_dot][key][query]
+    constexpr int oBT = SM::bounce_one, BBUF = (HAS_G ? 2 : 1) * SM::bounce_one;
     elem_t* ring = ownV + SM::vregion;
     elem_t* qstage = ring + R * SM::slot;                 // dQ (, dQ_dot) tiles of one stage on their way out
     // slot layout
     constexpr int oTQ = SE, oG = 2 * SE, oDO = (HAS_G ? 3 : 1) * SE;
     constexpr int oO = oDO + (HAS_DO ? SE : 0), oTO = oO + SE;
     constexpr int oST = SM::nt * SE;
-    constexpr int BP = SM::bpitch;
+    constexpr int BP = kStageRows;  // elements per key row of a bounce tile
     constexpr int KC = HD / 32;
     constexpr int DT = HD / 16;
 
     const int tid = threadIdx.x;
+    if (tid == 0) *reinterpret_cast<unsigned*>(smem_raw + SM::sink + 8) = 0u;  // see `announced` below
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
@@ -184,7 +193,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     }
 
     // Step 2: this wave's 32 x 16 tiles of one stage.
-    auto tile = [&](const elem_t* slot) {
+    auto tile = [&](const elem_t* slot, elem_t* bounceS) {
         const elem_t* sQ = slot;
         const elem_t* sTQ = slot + oTQ;
         const elem_t* sG = slot + oG;
@@ -266,15 +275,17 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             pdB = pack_b16<T>(ts[0], ts[1]);
             dtsB = pack_b16<T>(w[0], w[1]);
         }
-        // bounce[key][query]: the packed registers 2t, 2t+1 are queries 16t + 4g .. + 3 of key 16w + n
+        // bounce[key][query]: the packed registers 2t, 2t+1 are queries 16t + 4g .. + 3, i.e. unit 4t + g, of
+        // key 16w + n
         {
-            elem_t* bs = bounceS + (wave * 16 + n) * BP + 4 * g;
-            *reinterpret_cast<u32x2*>(bs) = u32x2{dsB[0], dsB[1]};
-            *reinterpret_cast<u32x2*>(bs + 16) = u32x2{dsB[2], dsB[3]};
+            const int key = wave * 16 + n;
+            elem_t* row = bounceS + key * BP;
+            const int u0 = (g ^ bounce_swz(key)) << 2, u1 = ((4 + g) ^ bounce_swz(key)) << 2;
+            *reinterpret_cast<u32x2*>(row + u0) = u32x2{dsB[0], dsB[1]};
+            *reinterpret_cast<u32x2*>(row + u1) = u32x2{dsB[2], dsB[3]};
             if constexpr (HAS_G) {
-                elem_t* bt = bounceT + (wave * 16 + n) * BP + 4 * g;
-                *reinterpret_cast<u32x2*>(bt) = u32x2{dtsB[0], dtsB[1]};
-                *reinterpret_cast<u32x2*>(bt + 16) = u32x2{dtsB[2], dtsB[3]};
+                *reinterpret_cast<u32x2*>(row + oBT + u0) = u32x2{dtsB[0], dtsB[1]};
+                *reinterpret_cast<u32x2*>(row + oBT + u1) = u32x2{dtsB[2], dtsB[3]};
             }
         }
 #pragma unroll
@@ -300,7 +311,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // the k numbering of lds_a_tr16 (rows 4g..4g+3 and 16+4g..16+4g+3 of the slab).
     auto bounce_b = [&](const elem_t* bounce, int kk, int qt) {
         const int i16 = lane & 15;
-        const elem_t* p0 = bounce + (32 * kk + 4 * g + (i16 >> 2)) * BP + 16 * qt + 4 * (i16 & 3);
+        const int row = 32 * kk + 4 * g + (i16 >> 2);  // rows row and row + 16 share their swizzle
+        const elem_t* p0 = bounce + row * BP + (((4 * qt + (i16 & 3)) ^ bounce_swz(row)) << 2);
         typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0));
         s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p0 + 16 * BP));
@@ -312,7 +324,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // Step 3: 16 x 16 tiles (head-dimension tile dt, query tile qt) of dQ and dQ_dot for the stage.
     // HD = 64: wave w forms tile w of both; HD = 32: waves 0..3 form dQ, waves 4..7 dQ_dot.
     constexpr int NTILES = 2 * DT;
-    auto row_outputs = [&](int row0, auto full_tag) {
+    auto row_outputs = [&](const elem_t* bounceS, elem_t* qstage_i, auto full_tag) {
+        const elem_t* bounceT = bounceS + oBT;
         constexpr bool FULL = decltype(full_tag)::value;  // all four key slabs hold keys
         const int tq = wave;                           // dQ tile of this wave
         const int tt = NTILES == 8 ? wave : wave - 4;      // dQ_dot tile of this wave
@@ -345,7 +358,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
         // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3: into the staging tile, from
         // where flush_rows() sends whole rows after the next barrier
-        elem_t* st = qstage + (16 * qt + n) * SM::qpitch + 16 * dt + 4 * g;
+        elem_t* st = qstage_i + (16 * qt + n) * SM::qpitch + 16 * dt + 4 * g;
         if (do_q) {
             a0 += a1;
             *reinterpret_cast<u32x2*>(st) =
@@ -359,13 +372,13 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // dQ (threads 0..255) and dQ_dot (256..511) of the stage that starts at row0: one 16-byte piece
     // of a row per thread (HD / 8 pieces per row).  Issued before the stage copy of the iteration, so
     // the stores are older than every copy a later wait_stages() still allows to be outstanding.
-    auto flush_rows = [&](int row0) {
+    auto flush_rows = [&](int row0, const elem_t* qstage_i) {
         constexpr int CH = HD / 8;
         const int half = tid >> 8, t = tid & 255;
         if (half == 1 && !HAS_G) return;
         const int r = t / CH, c = t % CH;
         if (r < kStageRows && row0 + r < p.Lq && 8 * c < p.D) {
-            const elem_t* srow = qstage + half * kStageRows * SM::qpitch + r * SM::qpitch;
+            const elem_t* srow = qstage_i + half * kStageRows * SM::qpitch + r * SM::qpitch;
             u32x4 v = *reinterpret_cast<const u32x4*>(srow + 8 * c);
             if constexpr (ROPE)
                 v = rope8_inverse_chunk<T>(v, *reinterpret_cast<const u32x4*>(srow + 8 * (c ^ 4)), p.rope, row0 + r, c);
@@ -423,14 +436,33 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         if constexpr (HAS_G)
             store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
     };
+    // One workgroup barrier per stage.  Iteration i: step 2 of stage i (tiles into bounce buffer i % 2), the
+    // barrier, then the row sums of stage i+1, step 3 of stage i (bounce buffer i % 2 -> staging buffer i % 2)
+    // and the rows of stage i-1 on their way out (staging buffer (i-1) % 2).  Step 2 of stage i+1 follows
+    // without a barrier: it writes the other bounce buffer, and what it needs from other waves, the
+    // statistics (and rotated rows) of stage i+1, is announced through a counter in LDS that the waves
+    // forming them raise (SIG waves per stage), which a wave polls before its step 2.
+    constexpr unsigned SIG = ROPE ? 8 : 4;
+    unsigned* announced = reinterpret_cast<unsigned*>(smem_raw + SM::sink + 8);
+    auto announce = [&]() {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // this wave's LDS writes are done
+        if (lane == 0) __hip_atomic_fetch_add(announced, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    auto await_announced = [&](unsigned target) {
+        // the announcing waves get there without waiting for anyone behind this point; the bound only
+        // keeps a mistake from hanging the machine
+        typedef __attribute__((address_space(3))) volatile unsigned lds_counter;  // an LDS read, not a flat one
+        lds_counter* flag = (lds_counter*)announced;
+        for (int spins = 0; *flag < target && spins < (1 << 22); ++spins) __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+    };
+    workgroup_barrier();  // every wave has read V, V_dot, whose memory the bounce tiles take over
     for (int i = 0; i < ns; ++i) {
-        // stage i and its statistics are visible; stage i-1 and the bounce tile are free (at i = 0
-        // every wave has read V, V_dot, whose memory the bounce tile takes over)
-        workgroup_barrier();
-        if (i >= 1) flush_rows((i - 1) * kStageRows);
         if (issued < ns && issued < i + R) issue_next();  // into the slot of stage issued - R <= i - 1
         elem_t* slot = ring + (i % R) * SM::slot;
-        if (wave_active) tile(slot);
+        elem_t* bounce_i = bounce0 + (i & 1) * BBUF;
+        if (i >= 1) await_announced(SIG * (unsigned)i);
+        if (wave_active) tile(slot, bounce_i);
         if (!ROPE && i == ns - 1 && wave_active) {
             // The gradients of this wave's keys are complete.  They leave now, while step 3 of the last stage
             // is still to come, through per-wave staging tiles in the two ring slots that no stage uses again
@@ -441,16 +473,19 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
             key_gradients(ring + ((i + 1 + (wave >> 2)) % R) * SM::slot + (wave & 3) * StoreStage16<HD>::elems);
         }
         if (i + 1 < ns) wait_stages<SPT>(issued - 2 - i);  // stage i+1 has landed (this wave's part)
-        workgroup_barrier();
+        workgroup_barrier();  // bounce buffer i % 2 is complete; stage i+1 is in LDS; stage i's slot is free
+        if (i >= 1) flush_rows((i - 1) * kStageRows, qstage + ((i - 1) & 1) * SM::qstage_one);
         if (i + 1 < ns) {
             row_sums(ring + ((i + 1) % R) * SM::slot);
             rotate_stage(ring + ((i + 1) % R) * SM::slot, (i + 1) * kStageRows);
+            if (ROPE || tid < 256) announce();
         }
-        if (key_slabs == 4) row_outputs(i * kStageRows, std::true_type{});
-        else row_outputs(i * kStageRows, std::false_type{});
+        elem_t* qstage_i = qstage + (i & 1) * SM::qstage_one;
+        if (key_slabs == 4) row_outputs(bounce_i, qstage_i, std::true_type{});
+        else row_outputs(bounce_i, qstage_i, std::false_type{});
     }
     workgroup_barrier();  // the last stage's dQ (, dQ_dot) tiles are in their staging tile; the ring is free
-    flush_rows((ns - 1) * kStageRows);
+    flush_rows((ns - 1) * kStageRows, qstage + ((ns - 1) & 1) * SM::qstage_one);
     if constexpr (ROPE) {
         static_assert(R * SM::slot >= kWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
         if (wave_active) key_gradients(ring + wave * StoreStage16<HD>::elems);
