@@ -108,7 +108,10 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                    p.D == HD && (issued + 1) * kStageRows <= p.Lk);
         ++issued;
     };
-    while (issued < R && issued < ns) issue_next();
+    // Stage 0 only for now: the loads of the own rows below are awaited by a wait for everything this wave has
+    // outstanding (the compiler cannot tell them from the stage copies), so the later stages are issued once
+    // the own rows are in registers and land under the first stage's arithmetic.
+    issue_next();
 
     // own rows as B operands; row sums s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O) from the
     // lane's 16-byte pieces, combined over the four lanes of a query
@@ -143,7 +146,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         }
     }
     const float lse2 = p.lse[so] * kLog2e;
-    const float mu = HAS_G ? p.mu[so] : 0.f;
+    float mu = HAS_G ? p.mu[so] : 0.f;
+    asm volatile("" : "+v"(mu));  // awaited here
+    while (issued < R && issued < ns) issue_next();
     // every row below Lr gets its workspace entries (zeros beyond Lq except lse2, which is finite): the
     // column-owned kernel, which runs after this one, stages 32-row groups
     if constexpr (!SECOND) {
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
         ++issued;
     };
-    while (issued < R && issued < ns) issue_next();
+    issue_next();  // stage 0 only for now, see bwd_row16_kernel
 
     u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
     load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
@@ -365,6 +370,16 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
         if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
     }
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {  // the own rows are awaited here
+        asm volatile("" : "+v"(kB[c]));
+        if constexpr (DO_K) asm volatile("" : "+v"(vB[c]));
+        if constexpr (HAS_G) {
+            asm volatile("" : "+v"(tkB[c]));
+            if constexpr (DO_K) asm volatile("" : "+v"(tvB[c]));
+        }
+    }
+    while (issued < R && issued < ns) issue_next();
     const float sl2 = p.scale * kLog2e;
     f32x4 dk[DT], dv[DT], dtk[DT], dtv[DT];
 #pragma unroll
@@ -616,7 +631,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
         }
         ++issued;
     };
-    while (issued < R && issued < ns) issue_next();
+    issue_next();  // stage 0 only for now, see bwd_row16_kernel
 
     u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
     load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
@@ -625,6 +640,12 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
         load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
         load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
     }
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {  // the own rows are awaited here
+        asm volatile("" : "+v"(kB[c]), "+v"(vB[c]));
+        if constexpr (HAS_G) asm volatile("" : "+v"(tkB[c]), "+v"(tvB[c]));
+    }
+    while (issued < R && issued < ns) issue_next();
     const float sl2 = p.scale * kLog2e;
     f32x4 dk[DH], dv[DH], dtk[DH], dtv[DH];
 #pragma unroll
