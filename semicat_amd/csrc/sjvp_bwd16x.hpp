@@ -145,9 +145,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
             s7d = group_sum(s7d);
         }
     }
-    const float lse2 = p.lse[so] * kLog2e;
+    float lse2 = p.lse[so] * kLog2e;
     float mu = HAS_G ? p.mu[so] : 0.f;
-    asm volatile("" : "+v"(mu));  // awaited here
+    asm volatile("" : "+v"(lse2), "+v"(mu), "+v"(s4), "+v"(s7d));  // every load so far is awaited here
     while (issued < R && issued < ns) issue_next();
     // every row below Lr gets its workspace entries (zeros beyond Lq except lse2, which is finite): the
     // column-owned kernel, which runs after this one, stages 32-row groups
