@@ -56,7 +56,7 @@ __device__ __forceinline__ int bounce_swz(int key) { return 4 * ((key >> 2) & 1)
 // prologue, each stage's Q, Q_dot slabs by the threads that do not form row sums), and the gradients
 // dQ, dQ_dot, dK, dK_dot go back through the inverse rotation on their way out (head dimension 64).
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, bool ROPE = false>
-__global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdParams p) {
+__global__ __launch_bounds__(kThreads16, HAS_G ? 2 : 4) void bwd_fused16_kernel(const BwdParams p) {
     static_assert(HD <= 64, "the accumulators of four gradients must fit the register file");
     static_assert(!ROPE || HD == 64, "the folded rotation covers a head dimension of 64");
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -96,6 +96,15 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // queries through the bounce tile as 0 * inf otherwise).  Wave-uniform flag, per-lane predicate.
     const bool ragged_keys = wave * 16 + 16 > p.Lk;
     const bool key_padded = wave * 16 + n >= p.Lk;
+    // Without the cotangent on TO a wave needs few enough registers for two workgroups per compute unit
+    // (four waves per SIMD, 128 registers), if the lane geometry of the steps outside step 2 is formed where
+    // it is used instead of being carried through the stage loop: there it comes from a lane id the
+    // compiler cannot see through.
+    auto lane_now = [&]() {
+        int v = lane;
+        if constexpr (!HAS_G) asm volatile("" : "+v"(v));
+        return v;
+    };
 
     using StagePlan = CopyPlan<HD, SM::nt, 1>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
@@ -150,7 +159,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // partial sums meet through DPP moves and the thread of column 0 writes the row's statistics.
     auto row_sums = [&](elem_t* slot) {
         if (tid >= 256) return;
-        const int r = tid >> 3, part = tid & 7;
+        const int tid_l = wave * 64 + lane_now();
+        const int r = tid_l >> 3, part = tid_l & 7;
         float s4 = 0.f, s7d = 0.f;
         if (part < HD / 8) {
             const int off = r * HD + ((part ^ swz<HD>(r)) << 3);
@@ -309,8 +319,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
 
     // B operand of step 3: Tile[k = key][x = query 16*qt + n] from a bounce tile, keys of slab kk in
     // the k numbering of lds_a_tr16 (rows 4g..4g+3 and 16+4g..16+4g+3 of the slab).
-    auto bounce_b = [&](const elem_t* bounce, int kk, int qt) {
-        const int i16 = lane & 15;
+    auto bounce_b = [&](const elem_t* bounce, int kk, int qt, int lane_l) {
+        const int i16 = lane_l & 15, g = lane_l >> 4;
         const int row = 32 * kk + 4 * g + (i16 >> 2);  // rows row and row + 16 share their swizzle
         const elem_t* p0 = bounce + row * BP + (((4 * qt + (i16 & 3)) ^ bounce_swz(row)) << 2);
         typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -334,20 +344,21 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         const int tile_id = do_q ? tq : tt;
         if (!do_q && !do_t) return;
         const int dt = tile_id % DT, qt = tile_id / DT;
+        const int lane_l = lane_now();
         // three independent chains: dS K, dS_dot K_dot (both into dQ) and dS_dot K (dQ_dot)
         f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
         auto step = [&](int kk) {
-            const u32x4 ak = lds_a_tr16<HD>(ownK + kk * SE, 16 * dt, lane);
+            const u32x4 ak = lds_a_tr16<HD>(ownK + kk * SE, 16 * dt, lane_l);
             if (do_q) {
-                a0 = T::mfma16(ak, bounce_b(bounceS, kk, qt), a0);
+                a0 = T::mfma16(ak, bounce_b(bounceS, kk, qt, lane_l), a0);
                 if constexpr (HAS_G) {
-                    const u32x4 bt = bounce_b(bounceT, kk, qt);
-                    const u32x4 atk = lds_a_tr16<HD>(ownK + (4 + kk) * SE, 16 * dt, lane);
+                    const u32x4 bt = bounce_b(bounceT, kk, qt, lane_l);
+                    const u32x4 atk = lds_a_tr16<HD>(ownK + (4 + kk) * SE, 16 * dt, lane_l);
                     a1 = T::mfma16(atk, bt, a1);
                     if (do_t) a2 = T::mfma16(ak, bt, a2);
                 }
             } else {
-                a2 = T::mfma16(ak, bounce_b(bounceT, kk, qt), a2);
+                a2 = T::mfma16(ak, bounce_b(bounceT, kk, qt, lane_l), a2);
             }
         };
         if constexpr (FULL) {
@@ -358,7 +369,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
         }
         // lane = query 16*qt + n, registers = columns 16*dt + 4g .. + 3: into the staging tile, from
         // where flush_rows() sends whole rows after the next barrier
-        elem_t* st = qstage_i + (16 * qt + n) * SM::qpitch + 16 * dt + 4 * g;
+        elem_t* st = qstage_i + (16 * qt + (lane_l & 15)) * SM::qpitch + 16 * dt + 4 * (lane_l >> 4);
         if (do_q) {
             a0 += a1;
             *reinterpret_cast<u32x2*>(st) =
@@ -374,7 +385,8 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_fused16_kernel(const BwdPar
     // the stores are older than every copy a later wait_stages() still allows to be outstanding.
     auto flush_rows = [&](int row0, const elem_t* qstage_i) {
         constexpr int CH = HD / 8;
-        const int half = tid >> 8, t = tid & 255;
+        const int tid_l = wave * 64 + lane_now();
+        const int half = tid_l >> 8, t = tid_l & 255;
         if (half == 1 && !HAS_G) return;
         const int r = t / CH, c = t % CH;
         if (r < kStageRows && row0 + r < p.Lq && 8 * c < p.D) {
