@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     // their absolute sums, which only set the scale of a threshold and are sampled on every fourth key.
     float r4 = 0.f, r7 = 0.f, a4 = 0.f, a7 = 0.f;
 
-    auto compute = [&](const elem_t* slot, int k0) {
+    auto compute = [&](const elem_t* slot, int k0, auto ragged_tag) {
         const elem_t* sK = slot;
         const elem_t* sV = slot + SE;
         const elem_t* sTK = slot + 2 * SE;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                 if constexpr (HAS_DO) xy[t] = T::mfma16(av, doB[c], xy[t]);
             }
         };
-        const bool ragged = k0 + kStageRows > p.Lk;  // wave-uniform: only the last stage
+        constexpr bool ragged = decltype(ragged_tag)::value;  // the stage reaches beyond Lk (only the last one can)
         // in place: w -> dS_dot, xy -> dS
         auto pointwise = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
@@ -201,7 +201,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                 float pj = fast_exp2(fmaf(s[t][j], sl2, -lse2));
                 // keys beyond Lk are zero rows; exp(-lse) may overflow when every real score is very
                 // negative, so their P is forced to zero
-                if (ragged && k0 + 16 * t + 4 * g + j >= p.Lk) pj = 0.f;
+                if constexpr (ragged) {
+                    if (k0 + 16 * t + 4 * g + j >= p.Lk) pj = 0.f;
+                }
                 if constexpr (HAS_G) {
                     const float nn = fmaf(ts[t][j], p.scale, -mu);
                     const float dts = pj * (w[t][j] - s4);
@@ -258,14 +260,18 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         }
     };
 
-    for (int i = 0; i < ns; ++i) {
+    // The last stage, the only one that can reach beyond Lk, runs behind the loop in a form of its own: the
+    // selects of its padded keys (a compare and two selects per tile element) stay out of the loop.
+    auto stage = [&](int i, auto ragged_tag) {
         // copies issued after stage i: the later stages; anything else in flight (the own rows'
         // loads, the statistics) only makes the wait stricter
         wait_stages<SPT>(issued - 1 - i);
         workgroup_barrier();  // stage i has landed for every wave; stage i-1 is fully consumed
         if (i > 0 && issued < ns) issue_next();
-        if (wave_active) compute(ring + (i % R) * SM::slot, i * kStageRows);
-    }
+        if (wave_active) compute(ring + (i % R) * SM::slot, i * kStageRows, ragged_tag);
+    };
+    for (int i = 0; i < ns - 1; ++i) stage(i, std::false_type{});
+    stage(ns - 1, std::true_type{});
     if constexpr (!SECOND) {
         // the residues of the row sums (see the top of the file); the four lanes of a query hold its keys
         r4 = group_sum(r4);
