@@ -1,7 +1,7 @@
 // Attention-JVP backward for key axes beyond one workgroup, 16-wide form (gfx950; inputs with 16-byte
-// aligned rows): the row-owned and column-owned pair of sjvp_bwd.hpp (same mathematics, same
-// workspace hand-over of lse*log2e, s4, s7d) with 16 owned positions per wavefront, so that several
-// wavefronts share a SIMD and a workgroup's copies overlap another's arithmetic.
+// aligned rows): the row-owned and column-owned pair of sjvp_bwd.hpp (same mathematics, the same
+// workspace arrays lse*log2e, s4, s7d, the two sums negated here) with 16 owned positions per wavefront,
+// so that several wavefronts share a SIMD and a workgroup's copies overlap another's arithmetic.
 //   bwd_row16_kernel   4 waves x 16 queries; streams K, V (, K_dot, V_dot)        -> dQ (, dQ_dot)
 //   bwd_col16_kernel   4 waves x 16 keys;    streams Q (, Q_dot, G) (, dO) + stats -> dK, dV (, dK_dot, dV_dot)
 // (workgroups of four waves: at 160-200 registers two or three of them share a CU)
@@ -16,7 +16,9 @@
 // residues in fp32 beside its tiles (per-lane adds) and
 //   - leaves the corrected sums s4' + rho4 = sum_j P W, s7d' + rho7 = sum_j P (N W + XY) in the
 //     workspace: the column-owned kernel works with the sums the reference's preprocess kernel forms
-//     from the probabilities (semicat/jvp_utils/flash_jvp_backward.py:2266-2287);
+//     from the probabilities (semicat/jvp_utils/flash_jvp_backward.py:2266-2287).  They are stored
+//     negated: both kernels start the accumulators of W and XY from minus the sums, so that W - s4 and
+//     XY - s7d come out of the matrix cores and cost no vector instruction;
 //   - flags its workgroup where a residue is not small against the row's |dS_dot| / |dS| mass (sharp
 //     rows, gradients formed by cancellation).  A second launch of the same kernel (PASS = 2) runs the
 //     flagged workgroups again with the corrected sums, so that their dQ, dQ_dot are formed from tiles
@@ -92,7 +94,20 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         if (p.rowfix == 1 && p.flags[bid] == 0) return;  // nothing to repair in this workgroup's rows
     }
 
-    // the ring first, so that the copies stream while the own rows are fetched
+    // The own rows are requested first, as B operands; the set-up of the stage copies runs while they travel.
+    u32x4 qB[KC], tqB[KC], gB[KC], doB[KC];
+    u32x4 oR[KC], toR[KC];
+    float s4 = 0.f, s7d = 0.f;
+    const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
+    load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
+    if constexpr (!SECOND) load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
+    if constexpr (HAS_G) {
+        load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
+        load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
+        if constexpr (!SECOND) load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
+    }
+    if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
+
     using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
     constexpr int SPT = StagePlan::N;
     StagePlan plan;
@@ -108,30 +123,18 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                    p.D == HD && (issued + 1) * kStageRows <= p.Lk);
         ++issued;
     };
-    // Stage 0 only for now: the loads of the own rows below are awaited by a wait for everything this wave has
+    // Stage 0 only for now: the loads of the own rows are awaited by a wait for everything this wave has
     // outstanding (the compiler cannot tell them from the stage copies), so the later stages are issued once
     // the own rows are in registers and land under the first stage's arithmetic.
     issue_next();
 
-    // own rows as B operands; row sums s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O) from the
-    // lane's 16-byte pieces, combined over the four lanes of a query
-    u32x4 qB[KC], tqB[KC], gB[KC], doB[KC];
-    float s4 = 0.f, s7d = 0.f;
-    const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
+    // row sums s4 = rowsum(G*O), s7d = rowsum(G*TO) + rowsum(dO*O) from the lane's 16-byte pieces, combined
+    // over the four lanes of a query
     {
-        u32x4 oR[KC], toR[KC];
-        load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
-        if constexpr (!SECOND) load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
-        if constexpr (HAS_G) {
-            load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
-            load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
-            if constexpr (!SECOND) load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
-        }
-        if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
         if constexpr (SECOND) {
-            // the corrected sums the first launch left in the workspace
-            s4 = p.s4[so];
-            s7d = p.s7d[so];
+            // the corrected sums the first launch left in the workspace (negated there)
+            s4 = -p.s4[so];
+            s7d = -p.s7d[so];
         } else {
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
@@ -147,7 +150,10 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     }
     float lse2 = p.lse[so] * kLog2e;
     float mu = HAS_G ? p.mu[so] : 0.f;
-    asm volatile("" : "+v"(lse2), "+v"(mu), "+v"(s4), "+v"(s7d));  // every load so far is awaited here
+    // The tiles W and XY are accumulated on top of -s4 and -s7d, so that W - s4 and XY - s7d leave the matrix
+    // cores ready for use.
+    float n4 = -s4, n7 = -s7d;
+    asm volatile("" : "+v"(lse2), "+v"(mu), "+v"(n4), "+v"(n7));  // every load so far is awaited here
     while (issued < R && issued < ns) issue_next();
     // every row below Lr gets its workspace entries (zeros beyond Lq except lse2, which is finite): the
     // column-owned kernel, which runs after this one, stages 32-row groups
@@ -175,8 +181,8 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         auto scores = [&](int t) __attribute__((always_inline)) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+            w[t] = f32x4{n4, n4, n4, n4};
+            xy[t] = f32x4{n7, n7, n7, n7};
 #pragma unroll
             for (int c = 0; c < KC; ++c) {
                 const u32x4 ak = lds_a_rows16<HD>(sK, t, c, n, g);
@@ -206,15 +212,15 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
                 }
                 if constexpr (HAS_G) {
                     const float nn = fmaf(ts[t][j], p.scale, -mu);
-                    const float dts = pj * (w[t][j] - s4);
+                    const float dts = pj * w[t][j];
                     w[t][j] = dts;
-                    xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s7d));
+                    xy[t][j] = fmaf(dts, nn, pj * xy[t][j]);
                     if constexpr (!SECOND) {
                         r4 += dts;
                         if (j == 0) a4 += fabsf(dts);
                     }
                 } else {
-                    xy[t][j] = pj * (xy[t][j] - s7d);
+                    xy[t][j] = pj * xy[t][j];
                 }
                 if constexpr (!SECOND) {
                     r7 += xy[t][j];
@@ -279,8 +285,8 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         a4 = 4.0f * group_sum(a4);
         a7 = 4.0f * group_sum(a7);
         if (g == 0) {
-            p.s4[so] = s4 + r4;
-            p.s7d[so] = s7d + r7;
+            p.s4[so] = n4 - r4;  // minus the corrected sums: the column-owned kernel starts its tiles from them
+            p.s7d[so] = n7 - r7;
         }
         // A residue matters where it is not small against the rounding of the tiles it is spread over:
         // |rho| against tau * sum_j |tile_ij|, tau = the unit roundoff of the 16-bit format.  NaN compares false.
@@ -340,6 +346,14 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (key0 + wave * 16) < p.Lk;
 
+    // the own rows are requested first; the set-up of the stage copies runs while they travel
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
+    if constexpr (DO_K) load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
+    if constexpr (HAS_G) {
+        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
+        if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+    }
     using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
     StagePlan plan;
@@ -369,13 +383,6 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     };
     issue_next();  // stage 0 only for now, see bwd_row16_kernel
 
-    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
-    if constexpr (DO_K) load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
-    if constexpr (HAS_G) {
-        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
-        if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
-    }
 #pragma unroll
     for (int c = 0; c < KC; ++c) {  // the own rows are awaited here
         asm volatile("" : "+v"(kB[c]));
@@ -433,20 +440,23 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
             return a;
         };
         f32x4 s[2], ts[2], w[2], xy[2];
-        f32x4 lse4[2], mu4[2], s44[2], s74[2];
+        f32x4 lse4[2], mu4[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
             ts[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            w[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            xy[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        auto load_stats = [&](int u) __attribute__((always_inline)) {
+        // The workspace holds -s4 and -s7d: W and XY are accumulated on top of them, so that W - s4 and
+        // XY - s7d leave the matrix cores ready for use.
+        auto load_sums = [&](int u) __attribute__((always_inline)) {
             const int r0 = 16 * u + 4 * g;  // register j of tile u is query 16 u + 4 g + j
+            if constexpr (HAS_G && DO_K) w[u] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+            if constexpr (DO_K) xy[u] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
+        };
+        auto load_stats = [&](int u) __attribute__((always_inline)) {
+            const int r0 = 16 * u + 4 * g;
             lse4[u] = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
             if constexpr (HAS_G) mu4[u] = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
-            if constexpr (HAS_G && DO_K) s44[u] = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
-            if constexpr (DO_K) s74[u] = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
         };
         auto score_step = [&](int t, int c, const AOps& a) __attribute__((always_inline)) {
             s[t] = T::mfma16(a.q, kB[c], s[t]);
@@ -470,21 +480,28 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
                 if constexpr (HAS_G) {
                     const float nn = fmaf(ts[t][j], p.scale, -mu4[t][j]);
                     if constexpr (DO_K) {
-                        const float dts = pj * (w[t][j] - s44[t][j]);
+                        const float dts = pj * w[t][j];
                         w[t][j] = dts;
-                        xy[t][j] = fmaf(dts, nn, pj * (xy[t][j] - s74[t][j]));
+                        xy[t][j] = fmaf(dts, nn, pj * xy[t][j]);
                     }
                     if constexpr (DO_V) ts[t][j] = pj * nn;
                 } else if constexpr (DO_K) {
-                    xy[t][j] = pj * (xy[t][j] - s74[t][j]);
+                    xy[t][j] = pj * xy[t][j];
                 }
             }
         };
+        load_sums(0);
         AOps cur = load_score(0, 0);
         load_stats(0);
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-            AOps nxt = c + 1 < KC ? load_score(0, c + 1) : load_score(1, 0);
+            AOps nxt;
+            if (c + 1 < KC) {
+                nxt = load_score(0, c + 1);
+            } else {
+                load_sums(1);
+                nxt = load_score(1, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of this step's MFMAs
             score_step(0, c, cur);
             __builtin_amdgcn_sched_barrier(0);
@@ -672,7 +689,11 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
         const elem_t* sG = slot + oG;
         const elem_t* sDO = slot + oDO;
         const float* sStat = reinterpret_cast<const float*>(slot + oST);
-        f32x4 s = {0.f, 0.f, 0.f, 0.f}, ts = {0.f, 0.f, 0.f, 0.f}, w = {0.f, 0.f, 0.f, 0.f}, xy = {0.f, 0.f, 0.f, 0.f};
+        // the workspace holds -s4 and -s7d: W and XY are accumulated on top of them
+        const int r0 = 16 * m + 4 * g;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, ts = {0.f, 0.f, 0.f, 0.f};
+        f32x4 w = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
+        f32x4 xy = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
             const u32x4 aq = lds_a_rows16<HD>(sQ, m, c, n, g);
@@ -691,23 +712,20 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
             }
         }
         // rows beyond Lq are zero rows of Q, Q_dot, G, dO with finite statistics: they contribute nothing
-        const int r0 = 16 * m + 4 * g;
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sStat + 0 * kStageRows + r0);
         const f32x4 mu4 = *reinterpret_cast<const f32x4*>(sStat + 1 * kStageRows + r0);
-        const f32x4 s44 = *reinterpret_cast<const f32x4*>(sStat + 2 * kStageRows + r0);
-        const f32x4 s74 = *reinterpret_cast<const f32x4*>(sStat + 3 * kStageRows + r0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float pj = fast_exp2(fmaf(s[j], sl2, -lse4[j]));
             s[j] = pj;
             if constexpr (HAS_G) {
                 const float nn = fmaf(ts[j], p.scale, -mu4[j]);
-                const float dts = pj * (w[j] - s44[j]);
+                const float dts = pj * w[j];
                 w[j] = dts;
-                xy[j] = fmaf(dts, nn, pj * (xy[j] - s74[j]));
+                xy[j] = fmaf(dts, nn, pj * xy[j]);
                 ts[j] = pj * nn;
             } else {
-                xy[j] = pj * (xy[j] - s74[j]);
+                xy[j] = pj * xy[j];
             }
         }
         mine[0] = u32x2{T::pack2(s[0], s[1]), T::pack2(s[2], s[3])};
