@@ -206,6 +206,20 @@ int run_bwd(int parts, const BwdTensors& t, float* ws, int B, int H, int Lq, int
     p.scale = resolve_scale(scale, D);
     p.vec = (vc.ok && D % 8 == 0) ? 1 : 0;
     p.rope = rope;
+    {
+        auto same = [&](int a, int b) {
+            return !ptrs[b] || (strides[3 * a] == strides[3 * b] && strides[3 * a + 1] == strides[3 * b + 1] &&
+                                strides[3 * a + 2] == strides[3 * b + 2]);
+        };
+        auto fits = [&](int a, int rows) {
+            return strides[3 * a + 2] >= 0 && (int64_t)rows * strides[3 * a + 2] + D < (int64_t(1) << 29);
+        };
+        p.q_side_uniform = !f32io && fits(SJVP_B_Q, p.Lr) && same(SJVP_B_Q, SJVP_B_TQ) && same(SJVP_B_Q, SJVP_B_O) &&
+                           same(SJVP_B_Q, SJVP_B_TO) && (!has_do || same(SJVP_B_Q, SJVP_B_DO)) &&
+                           (!has_g || same(SJVP_B_Q, SJVP_B_DTO));
+        p.k_side_uniform = !f32io && fits(SJVP_B_K, round_up(Lk, kOwned)) && same(SJVP_B_K, SJVP_B_V) &&
+                           same(SJVP_B_K, SJVP_B_TK) && same(SJVP_B_K, SJVP_B_TV);
+    }
     p.rowfix = g_row_sum_repair.load(std::memory_order_relaxed);
     p.rowfix_tau = dtype == SJVP_FP16 ? 0x1p-11f : 0x1p-8f;  // unit roundoff of the tiles' 16-bit format
     if (rope.cos && (!p.vec || parts != SJVP_BWD_ALL)) return SJVP_ERR_ROTARY;  // the single launch only

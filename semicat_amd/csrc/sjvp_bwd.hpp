@@ -37,6 +37,10 @@ struct BwdParams {
     float* s7d;   // workspace [B*H][Lr]  rowsum(G*TO) + rowsum(dO*O)
     int H, Lq, Lk, D, Lr;
     int q_blocks, k_blocks;  // workgroups per (batch, head) along the owned axis
+    // Set by the host where every query-side input (q, q_dot, o, o_dot, dO, dO_dot as present) has q's strides,
+    // resp. every key-side input k's, and a row's byte offset inside its (batch, head) slice fits 31 bits: the
+    // 16-wide row-owned and column-owned kernels then address their own rows from one offset.
+    int q_side_uniform, k_side_uniform;
     float scale;
     int vec;
     RopeTables rope;  // q, k (and tangents) are rotated as they are loaded, their gradients rotated back

@@ -42,6 +42,15 @@ __device__ __forceinline__ void load_b_operands16(u32x4* out, const elem_t* row,
     for (int c = 0; c < HD / 32; ++c) out[c] = load8(row, 32 * c + 8 * g, D, valid, true);
 }
 
+// The same from a uniform slice pointer and the lane's byte offset in the slice: whole rows of HD elements
+// that all exist, no predicates, one 32-bit offset for every tensor of equal strides.
+template <int HD>
+__device__ __forceinline__ void load_b_operands16_at(u32x4* out, const elem_t* slice, uint32_t lane_bytes) {
+    const char* base = reinterpret_cast<const char*>(slice);
+#pragma unroll
+    for (int c = 0; c < HD / 32; ++c) out[c] = *reinterpret_cast<const u32x4*>(base + lane_bytes + 64 * c);
+}
+
 // sum over the 16-bit pairs of a[i]*b[i]
 template <typename T>
 __device__ __forceinline__ float dot8(const u32x4& a, const u32x4& b) {
@@ -99,14 +108,30 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     u32x4 oR[KC], toR[KC];
     float s4 = 0.f, s7d = 0.f;
     const int64_t so = (int64_t)bh * p.Lr + qrow;  // rows below Lr exist in every statistic
-    load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
-    if constexpr (!SECOND) load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
-    if constexpr (HAS_G) {
-        load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
-        load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
-        if constexpr (!SECOND) load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
+    if (p.q_side_uniform && p.D == HD && q0 + kXOwned16 <= p.Lq) {
+        // the common case: whole rows that all exist, every tensor with q's strides
+        const int64_t slice = b * p.q.sb + h * p.q.sh;
+        const uint32_t at = ((uint32_t)qrow * (uint32_t)p.q.sl + 8u * (uint32_t)g) * (uint32_t)sizeof(elem_t);
+        load_b_operands16_at<HD>(qB, p.q.ptr + slice, at);
+        if constexpr (!SECOND) load_b_operands16_at<HD>(oR, p.o.ptr + slice, at);
+        if constexpr (HAS_G) {
+            load_b_operands16_at<HD>(tqB, p.tq.ptr + slice, at);
+            load_b_operands16_at<HD>(gB, p.dTO.ptr + slice, at);
+            if constexpr (!SECOND) load_b_operands16_at<HD>(toR, p.to.ptr + slice, at);
+        }
+        if constexpr (HAS_DO) load_b_operands16_at<HD>(doB, p.dO.ptr + slice, at);
+    } else {
+        load_b_operands16<HD>(qB, p.q.head(b, h) + (int64_t)qrow * p.q.sl, g, p.D, qvalid);
+        if constexpr (!SECOND) load_b_operands16<HD>(oR, p.o.head(b, h) + (int64_t)qrow * p.o.sl, g, p.D, qvalid);
+        if constexpr (HAS_G) {
+            load_b_operands16<HD>(tqB, p.tq.head(b, h) + (int64_t)qrow * p.tq.sl, g, p.D, qvalid);
+            load_b_operands16<HD>(gB, p.dTO.head(b, h) + (int64_t)qrow * p.dTO.sl, g, p.D, qvalid);
+            if constexpr (!SECOND) load_b_operands16<HD>(toR, p.to.head(b, h) + (int64_t)qrow * p.to.sl, g, p.D, qvalid);
+        }
+        if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
     }
-    if constexpr (HAS_DO) load_b_operands16<HD>(doB, p.dO.head(b, h) + (int64_t)qrow * p.dO.sl, g, p.D, qvalid);
+    float lse_in = p.lse[so];  // requested with the rows: they are awaited together
+    float mu_in = HAS_G ? p.mu[so] : 0.f;
 
     using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
     constexpr int SPT = StagePlan::N;
@@ -148,8 +173,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
             s7d = group_sum(s7d);
         }
     }
-    float lse2 = p.lse[so] * kLog2e;
-    float mu = HAS_G ? p.mu[so] : 0.f;
+    asm volatile("" : "+v"(lse_in), "+v"(mu_in));  // not before the copies of stage 0 are under way
+    float lse2 = lse_in * kLog2e;
+    float mu = HAS_G ? mu_in : 0.f;
     // The tiles W and XY are accumulated on top of -s4 and -s7d, so that W - s4 and XY - s7d leave the matrix
     // cores ready for use.
     float n4 = -s4, n7 = -s7d;
@@ -346,28 +372,9 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     const bool kvalid = krow < p.Lk;
     const bool wave_active = (key0 + wave * 16) < p.Lk;
 
-    // the own rows are requested first; the set-up of the stage copies runs while they travel
-    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
-    if constexpr (DO_K) load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
-    if constexpr (HAS_G) {
-        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
-        if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
-    }
     using StagePlan = CopyPlan<HD, SM::nt, 1, kXThreads16>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics
     StagePlan plan;
-    {
-        const Src q{p.q.head(b, h), p.q.sl};
-        if constexpr (HAS_G && HAS_DO)
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
-                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
-        else if constexpr (HAS_G)
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
-                      Src{p.dTO.head(b, h), p.dTO.sl});
-        else
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
-    }
     const int ns = (p.Lq + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
@@ -381,8 +388,44 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
         ++issued;
     };
-    issue_next();  // stage 0 only for now, see bwd_row16_kernel
-
+    // called behind the requests for the own rows on both paths below (see bwd_row16_kernel): set-up of the
+    // stage copies, and stage 0 only for now
+    auto begin_copies = [&]() __attribute__((always_inline)) {
+        {
+            const Src q{p.q.head(b, h), p.q.sl};
+            if constexpr (HAS_G && HAS_DO)
+                plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                          Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
+            else if constexpr (HAS_G)
+                plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                          Src{p.dTO.head(b, h), p.dTO.sl});
+            else
+                plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
+        }
+        issue_next();
+    };
+    // the own rows are requested first; the set-up of the stage copies runs while they travel
+    u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
+    if (p.k_side_uniform && p.D == HD && key0 + kXOwned16 <= p.Lk) {
+        // the common case: whole rows that all exist, every tensor with k's strides
+        const int64_t slice = b * p.k.sb + h * p.k.sh;
+        const uint32_t at = ((uint32_t)krow * (uint32_t)p.k.sl + 8u * (uint32_t)g) * (uint32_t)sizeof(elem_t);
+        load_b_operands16_at<HD>(kB, p.k.ptr + slice, at);
+        if constexpr (DO_K) load_b_operands16_at<HD>(vB, p.v.ptr + slice, at);
+        if constexpr (HAS_G) {
+            load_b_operands16_at<HD>(tkB, p.tk.ptr + slice, at);
+            if constexpr (DO_K) load_b_operands16_at<HD>(tvB, p.tv.ptr + slice, at);
+        }
+        begin_copies();
+    } else {
+        load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
+        if constexpr (DO_K) load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
+        if constexpr (HAS_G) {
+            load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
+            if constexpr (DO_K) load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+        }
+        begin_copies();
+    }
 #pragma unroll
     for (int c = 0; c < KC; ++c) {  // the own rows are awaited here
         asm volatile("" : "+v"(kB[c]));
@@ -627,17 +670,6 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
     using StagePlan = CopyPlan<HD, SM::nt, 1, kThreads16>;
     constexpr int SPT = StagePlan::N + 1;  // plus one 4-byte copy of statistics (or its placeholder)
     StagePlan plan;
-    {
-        const Src q{p.q.head(b, h), p.q.sl};
-        if constexpr (HAS_G && HAS_DO)
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
-                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
-        else if constexpr (HAS_G)
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
-                      Src{p.dTO.head(b, h), p.dTO.sl});
-        else
-            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
-    }
     const int ns = (p.Lq + kStageRows - 1) / kStageRows;
     int issued = 0;
     auto issue_next = [&]() {
@@ -654,14 +686,41 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
         }
         ++issued;
     };
-    issue_next();  // stage 0 only for now, see bwd_row16_kernel
-
+    // called behind the requests for the own rows on both paths below (see bwd_row16_kernel): set-up of the
+    // stage copies, and stage 0 only for now
+    auto begin_copies = [&]() __attribute__((always_inline)) {
+        const Src q{p.q.head(b, h), p.q.sl};
+        if constexpr (HAS_G && HAS_DO)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl}, Src{p.dO.head(b, h), p.dO.sl});
+        else if constexpr (HAS_G)
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.tq.head(b, h), p.tq.sl},
+                      Src{p.dTO.head(b, h), p.dTO.sl});
+        else
+            plan.init(tid, 0, p.D, smem_raw + SM::sink, q, Src{p.dO.head(b, h), p.dO.sl});
+        issue_next();
+    };
+    // the own rows are requested first; the set-up of the stage copies runs while they travel
     u32x4 kB[KC], vB[KC], tkB[KC], tvB[KC];
-    load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
-    load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
-    if constexpr (HAS_G) {
-        load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
-        load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+    if (p.k_side_uniform && p.D == HD && key0 + kXOwned16 <= p.Lk) {
+        // the common case: whole rows that all exist, every tensor with k's strides
+        const int64_t slice = b * p.k.sb + h * p.k.sh;
+        const uint32_t at = ((uint32_t)krow * (uint32_t)p.k.sl + 8u * (uint32_t)g) * (uint32_t)sizeof(elem_t);
+        load_b_operands16_at<HD>(kB, p.k.ptr + slice, at);
+        load_b_operands16_at<HD>(vB, p.v.ptr + slice, at);
+        if constexpr (HAS_G) {
+            load_b_operands16_at<HD>(tkB, p.tk.ptr + slice, at);
+            load_b_operands16_at<HD>(tvB, p.tv.ptr + slice, at);
+        }
+        begin_copies();
+    } else {
+        load_b_operands16<HD>(kB, p.k.head(b, h) + (int64_t)krow * p.k.sl, g, p.D, kvalid);
+        load_b_operands16<HD>(vB, p.v.head(b, h) + (int64_t)krow * p.v.sl, g, p.D, kvalid);
+        if constexpr (HAS_G) {
+            load_b_operands16<HD>(tkB, p.tk.head(b, h) + (int64_t)krow * p.tk.sl, g, p.D, kvalid);
+            load_b_operands16<HD>(tvB, p.tv.head(b, h) + (int64_t)krow * p.tv.sl, g, p.D, kvalid);
+        }
+        begin_copies();
     }
 #pragma unroll
     for (int c = 0; c < KC; ++c) {  // the own rows are awaited here
