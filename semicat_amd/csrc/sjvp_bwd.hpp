@@ -41,6 +41,7 @@ struct BwdParams {
     // resp. every key-side input k's, and a row's byte offset inside its (batch, head) slice fits 31 bits: the
     // 16-wide row-owned and column-owned kernels then address their own rows from one offset.
     int q_side_uniform, k_side_uniform;
+    int col_workgroups;  // workgroups of the column-owned pass in a launch that also holds others (set by its launcher)
     float scale;
     int vec;
     RopeTables rope;  // q, k (and tangents) are rotated as they are loaded, their gradients rotated back

@@ -72,8 +72,10 @@ struct Row16Smem {
     static_assert(R * slot >= kXWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC, int PASS = 0>
-__global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdParams p) {
+// (the body of the kernel as a function of the workgroup's index and the number of workgroups, so that the
+// second launch can also ride at the end of the column-owned launch, see bwd_col16_repair_kernel)
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int PASS>
+__device__ __forceinline__ void bwd_row16_body(const BwdParams p, const int block, const int blocks) {
     constexpr bool SECOND = PASS == 2;   // second launch: sums from the workspace, flagged workgroups only
     constexpr bool MEASURE = PASS == 1;  // first launch of "always": residues and sums only, no gradients
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
     // Workgroups run through the heads in descending order: this launch follows the forward, which
     // ran through them in ascending order, so it starts on what the caches still hold (the
     // column-owned launch after it ascends again).
-    const int bid = (int)gridDim.x - 1 - xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
+    const int bid = blocks - 1 - xcd_linear_id(block, blocks);
     const int bh = bid / q_blocks;
     const int qb = bid % q_blocks;
     const int b = bh / p.H, h = bh % p.H;
@@ -332,6 +334,11 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdPa
         store_tile16<T, HD>(stage_tile, p.dtq.head(b, h), p.dtq.sl, row0, p.Lq, p.D, dtq, p.scale, lane);
 }
 
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC, int PASS = 0>
+__global__ __launch_bounds__(kXThreads16, OCC) void bwd_row16_kernel(const BwdParams p) {
+    bwd_row16_body<T, HD, R, HAS_DO, HAS_G, PASS>(p, (int)blockIdx.x, (int)gridDim.x);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Column-owned kernel: a workgroup of four waves owns 64 keys.  PART selects the gradients that are
 // accumulated: 3 all four (HD <= 64), 1 dK (, dK_dot), 2 dV (, dV_dot) (HD = 128 runs as two launches
@@ -347,8 +354,8 @@ struct Col16Smem {
     static_assert(R * slot >= kXWaves16 * StoreStage16<HD>::elems, "ring too small to stage stores");
 };
 
-template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int PART, int OCC>
-__global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdParams p) {
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int PART>
+__device__ __forceinline__ void bwd_col16_body(const BwdParams p, const int block, const int blocks) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     using SM = Col16Smem<HD, R, HAS_DO, HAS_G>;
     constexpr bool DO_K = (PART & 1) != 0, DO_V = (PART & 2) != 0;
@@ -363,7 +370,7 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
     const int n = lane & 15;
     const int g = lane >> 4;
     const int k_blocks = (p.Lk + kXOwned16 - 1) / kXOwned16;
-    const int bid = xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
+    const int bid = xcd_linear_id(block, blocks);
     const int bh = bid / k_blocks;
     const int kb = bid % k_blocks;
     const int b = bh / p.H, h = bh % p.H;
@@ -383,7 +390,11 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         plan.issue(slot, p.Lq - row0, p.D == HD && row0 + kStageRows <= p.Lq);
         // the four statistic arrays (lse2, mu, s4, s7d) of the stage's rows, one per wave, 32 lanes
         // each (rows < Lr exist in all of them); every wave issues exactly one 4-byte LDS-DMA
-        const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;
+        // (the three workspace arrays lie one behind the other: chosen by arithmetic, which stays in scalar
+        // registers, where a choice among four pointers becomes a table in memory)
+        const int64_t plane = p.s4 - p.lse2;
+        const float* src = p.lse2 + (wave == 0 ? 0 : wave == 3 ? 2 : 1) * plane;  // lse2 | s4 | s4 | s7d
+        if (HAS_G && wave == 1) src = p.mu;
         float* st = reinterpret_cast<float*>(slot + oST);
         if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
         ++issued;
@@ -617,6 +628,25 @@ __global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdPa
         if constexpr (HAS_G)
             store_tile16<T, HD>(stage_tile, p.dtv.head(b, h), p.dtv.sl, row0, p.Lk, p.D, dtv, 1.0f, lane);
     }
+}
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int PART, int OCC>
+__global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_kernel(const BwdParams p) {
+    bwd_col16_body<T, HD, R, HAS_DO, HAS_G, PART>(p, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// The column-owned launch with the second launch of the row-owned kernel at its end: workgroups
+// 0 .. col_blocks - 1 are the column-owned kernel's, the rest the row-owned kernel's second pass, which does
+// not depend on the column pass (it rewrites dQ, dQ_dot of flagged workgroups from the sums the first pass
+// left).  Nearly all of those workgroups leave at once; dealt out behind the column pass they fill the time in
+// which its last workgroups run alone, where a launch of their own costs a few microseconds.
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G, int OCC>
+__global__ __launch_bounds__(kXThreads16, OCC) void bwd_col16_repair_kernel(const BwdParams p) {
+    const int col_blocks = p.col_workgroups;
+    if ((int)blockIdx.x < col_blocks)
+        bwd_col16_body<T, HD, R, HAS_DO, HAS_G, 3>(p, (int)blockIdx.x, col_blocks);
+    else
+        bwd_row16_body<T, HD, R, HAS_DO, HAS_G, 2>(p, (int)blockIdx.x - col_blocks, (int)gridDim.x - col_blocks);
 }
 
 // ---------------------------------------------------------------------------------------------

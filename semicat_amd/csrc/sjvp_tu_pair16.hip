@@ -15,6 +15,7 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
     // the column-owned one; workgroups of four waves own 64 positions
     constexpr int XR = HD == 128 ? 2 : 3;  // ring depth
     int rc = SJVP_OK;
+    bool rides = false;
     if (parts & SJVP_BWD_ROW) {
         constexpr int OCC = HD == 128 ? 2 : 3;
         const int grid = BH * (p.Lr / kXOwned16);
@@ -24,7 +25,11 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         // whose residues call for it run again
         if (p.rowfix == 2) rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 1>, grid, smem, stream, p, kXThreads16);
         else rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 0>, grid, smem, stream, p, kXThreads16);
-        if (rc == SJVP_OK && p.rowfix != 0)
+        // The second launch does not depend on the column-owned pass.  Where nearly all of its workgroups leave
+        // at once (repair of flagged workgroups only) and the column-owned kernel has the same workgroup size,
+        // they ride at the end of that launch instead of paying for one of their own.
+        rides = HD != 128 && p.rowfix == 1 && (parts & SJVP_BWD_COL);
+        if (rc == SJVP_OK && p.rowfix != 0 && !rides)
             rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 2>, grid, smem, stream, p, kXThreads16);
     }
     if (rc != SJVP_OK || !(parts & SJVP_BWD_COL)) return rc;
@@ -37,6 +42,13 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         return launch(bwd_col16p_kernel<T, HD, PR, HAS_DO, HAS_G>, grid, Col16pSmem<HD, PR, HAS_DO, HAS_G>::bytes,
                       stream, p, kThreads16);
     } else {
+        if (rides) {
+            BwdParams pr = p;
+            pr.col_workgroups = grid;
+            constexpr int smem = CS::bytes > Row16Smem<HD, XR, HAS_G>::bytes ? CS::bytes : Row16Smem<HD, XR, HAS_G>::bytes;
+            return launch(bwd_col16_repair_kernel<T, HD, XR, HAS_DO, HAS_G, 2>, grid + BH * (p.Lr / kXOwned16), smem,
+                          stream, pr, kXThreads16);
+        }
         return launch(bwd_col16_kernel<T, HD, XR, HAS_DO, HAS_G, 3, 2>, grid, CS::bytes, stream, p, kXThreads16);
     }
 }
