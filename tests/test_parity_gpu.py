@@ -149,6 +149,42 @@ def test_caller_layout_strided_views(K):
     assert_parity(res, ref, TOL_16BIT, label="strided")
 
 
+@pytest.mark.parametrize("L,D", [(256, 64), (192, 128), (320, 32)])
+@pytest.mark.parametrize("layout", ["mixed", "padded_rows", "all_seq_major"])
+def test_row_and_column_kernels_with_equal_and_unequal_strides(K, L, D, layout):
+    """The row-owned and column-owned kernels address the rows they own from one offset where every tensor
+    of a side has the same strides, and tensor by tensor otherwise; the host decides.  `mixed`: q-side and
+    k-side tensors in different layouts (o, to come head-major from the forward, v, v_dot head-major, the
+    rest sequence-major); `padded_rows`: every tensor with a row stride of D + 8 elements (equal strides that
+    are not the contiguous ones); `all_seq_major`: equal strides, sequence-major."""
+    B, H = 2, 3
+    x = orc.make_inputs(B, H, L, L, D, seed=21, dtype=torch.bfloat16)
+    ref = orc.attention_jvp_autograd(*[x[n] for n in orc.TENSOR_ORDER])
+    seq = lambda t: t.cuda().transpose(1, 2).contiguous().transpose(1, 2)
+
+    def padded(t):
+        buf = torch.zeros(B, H, L, D + 8, dtype=t.dtype, device="cuda")
+        buf[..., :D] = t.cuda()
+        return buf[..., :D]
+
+    if layout == "mixed":
+        d = {n: (t.cuda() if n in ("v", "tv") else seq(t)) for n, t in x.items()}
+    elif layout == "padded_rows":
+        d = {n: padded(t) for n, t in x.items()}
+        assert d["q"].stride() == (H * L * (D + 8), L * (D + 8), D + 8, 1)
+    else:
+        d = {n: seq(t) for n, t in x.items()}
+    o, to, lse, mu, li = K.attention_jvp_forward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"])
+    if layout == "padded_rows":
+        o, to = padded(o), padded(to)
+    elif layout == "all_seq_major":
+        o, to = seq(o), seq(to)
+    g = K.attention_jvp_backward(d["q"], d["k"], d["v"], d["tq"], d["tk"], d["tv"], o, to, lse, mu,
+                                 dO=d["dO"], dTO=d["dTO"])
+    res = {"O": o.cpu(), "TO": to.cpu(), **{n: t.cpu() for n, t in zip(GRADS, g)}}
+    assert_parity(res, ref, TOL_16BIT, label=f"{layout} L{L} D{D}")
+
+
 def test_unaligned_and_odd_head_dim_take_the_scalar_path(K):
     """D = 20 (not a multiple of 8) and a base pointer offset by one element."""
     B, H, L, D = 1, 2, 50, 20
