@@ -107,7 +107,10 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
  * sjvp_bwd_parts() runs the selected launches of that pair with sjvp_bwd()'s arguments;
  * sjvp_bwd_parts(SJVP_BWD_ALL, ...) is sjvp_bwd().  It has no counterpart in the reference: it exists
  * so that a profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only
- * valid on a workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.
+ * valid on a workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.  (The second
+ * pass of the row-owned kernel, see sjvp_set_row_sum_repair, belongs to SJVP_BWD_ROW; with SJVP_BWD_ALL its
+ * workgroups are appended to the column-owned launch where the two kernels' workgroups have one size, D <= 64,
+ * since it depends on the first row-owned launch only.)
  */
 enum sjvp_bwd_part { SJVP_BWD_ROW = 1, SJVP_BWD_COL = 2, SJVP_BWD_ALL = 3 };
 int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const void* tq,
@@ -171,10 +174,10 @@ int sjvp_bwd_noalloc(const void* q, const void* k, const void* v, const void* tq
  * This library takes all of them from the 16-bit outputs o, to, which costs no pass, and the
  * row-owned launch then measures what the rounding of o, to left in them (the sums over the keys of
  * dS_dot and of dS, zero in exact arithmetic): it hands the column-owned launch the corrected sums
- * (= the reference's sums), and a second launch of the row-owned kernel recomputes dq, dtq with them
- * for the workgroups that ask for it.
- *   SJVP_REPAIR_OFF     no second launch (dk, dtk still get the corrected sums)
- *   SJVP_REPAIR_AUTO    (default) the second launch runs the workgroups in which a row's residue exceeds
+ * (= the reference's sums), and a second pass of the row-owned kernel (a launch of its own, or workgroups
+ * appended to the column-owned launch) recomputes dq, dtq with them for the workgroups that ask for it.
+ *   SJVP_REPAIR_OFF     no second pass (dk, dtk still get the corrected sums)
+ *   SJVP_REPAIR_AUTO    (default) the second pass runs the workgroups in which a row's residue exceeds
  *                       the rounding of the tiles it is spread over (sharp attention rows, gradients
  *                       formed by cancellation); the others leave at once
  *   SJVP_REPAIR_ALWAYS  the first launch only measures, the second computes every row with the
@@ -191,7 +194,7 @@ int sjvp_set_row_sum_repair(int mode);
 /* Bytes of caller-provided device scratch sjvp_bwd needs: lse in log2 units and the row sums sum_4
  * and sum_7 + delta (the reference allocates sum_4, sum_7 and delta itself,
  * flash_jvp_backward.py:2355-2356 and flash_attn_triton.py:990), 12 bytes per statistic row, and one
- * 4-byte flag per 64 rows (which row-owned workgroups take the second launch of the repair below). */
+ * 4-byte flag per 64 rows (which row-owned workgroups take the second pass of the repair below). */
 size_t sjvp_bwd_workspace_bytes(int B, int H, int Lq, int Lk, int D, int dtype);
 
 /*
