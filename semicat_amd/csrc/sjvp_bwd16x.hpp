@@ -671,7 +671,7 @@ struct Col16pSmem {
 };
 
 template <typename T, int HD, int R, bool HAS_DO, bool HAS_G>
-__global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdParams p) {
+__device__ __forceinline__ void bwd_col16p_body(const BwdParams p, const int block, const int blocks) {
     static_assert(HD == 128, "the paired form exists for the head dimension that needs it");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     using SM = Col16pSmem<HD, R, HAS_DO, HAS_G>;
@@ -688,7 +688,7 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
     const int n = lane & 15;
     const int g = lane >> 4;
     const int k_blocks = (p.Lk + kXOwned16 - 1) / kXOwned16;
-    const int bid = xcd_linear_id((int)blockIdx.x, (int)gridDim.x);
+    const int bid = xcd_linear_id(block, blocks);
     const int bh = bid / k_blocks;
     const int kb = bid % k_blocks;
     const int b = bh / p.H, h = bh % p.H;
@@ -708,7 +708,9 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
         plan.issue(slot, p.Lq - row0, p.D == HD && row0 + kStageRows <= p.Lq);
         // the four statistic arrays of the stage's rows by waves 0..3; the others issue a placeholder
         if (wave < 4) {
-            const float* src = wave == 0 ? p.lse2 : wave == 1 ? (HAS_G ? p.mu : p.s4) : wave == 2 ? p.s4 : p.s7d;
+            const int64_t plane = p.s4 - p.lse2;  // see bwd_col16_body
+            const float* src = p.lse2 + (wave == 0 ? 0 : wave == 3 ? 2 : 1) * plane;  // lse2 | s4 | s4 | s7d
+            if (HAS_G && wave == 1) src = p.mu;
             float* st = reinterpret_cast<float*>(slot + oST);
             if (lane < 32) dma4(src + (int64_t)bh * p.Lr + row0 + lane, lds_addr(st) + (uint32_t)(wave * 32 * 4));
         } else {
@@ -886,6 +888,25 @@ __global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdPara
     store_tile16<T, 64>(stage_tile, p.dv.head(b, h) + dcol, p.dv.sl, row0, p.Lk, Dm, dv, 1.0f, lane);
     if constexpr (HAS_G)
         store_tile16<T, 64>(stage_tile, p.dtv.head(b, h) + dcol, p.dtv.sl, row0, p.Lk, Dm, dtv, 1.0f, lane);
+}
+
+template <typename T, int HD, int R, bool HAS_DO, bool HAS_G>
+__global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_kernel(const BwdParams p) {
+    bwd_col16p_body<T, HD, R, HAS_DO, HAS_G>(p, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// The paired column-owned launch with the second pass of the row-owned kernel at its end (see
+// bwd_col16_repair_kernel).  The row-owned kernel's workgroups have four waves, these eight: in a workgroup that
+// takes a row item the upper four leave at once, and the barriers of the others count the waves that are left.
+template <typename T, int HD, int R, int RROW, bool HAS_DO, bool HAS_G>
+__global__ __launch_bounds__(kThreads16, 2) void bwd_col16p_repair_kernel(const BwdParams p) {
+    const int col_blocks = p.col_workgroups;
+    if ((int)blockIdx.x < col_blocks) {
+        bwd_col16p_body<T, HD, R, HAS_DO, HAS_G>(p, (int)blockIdx.x, col_blocks);
+    } else {
+        if ((int)threadIdx.x >= kXThreads16) return;
+        bwd_row16_body<T, HD, RROW, HAS_DO, HAS_G, 2>(p, (int)blockIdx.x - col_blocks, (int)gridDim.x - col_blocks);
+    }
 }
 
 }  // namespace sjvp

@@ -26,9 +26,11 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         if (p.rowfix == 2) rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 1>, grid, smem, stream, p, kXThreads16);
         else rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 0>, grid, smem, stream, p, kXThreads16);
         // The second launch does not depend on the column-owned pass.  Where nearly all of its workgroups leave
-        // at once (repair of flagged workgroups only) and the column-owned kernel has the same workgroup size,
-        // they ride at the end of that launch instead of paying for one of their own.
-        rides = HD != 128 && p.rowfix == 1 && (parts & SJVP_BWD_COL);
+        // at once (repair of flagged workgroups only), they ride at the end of that launch instead of paying for
+        // one of their own.
+        // (not at D = 128 with the cotangent on O only: the row-owned body needs more registers than that
+        // column-owned kernel, which would lose a resident workgroup per compute unit to it)
+        rides = p.rowfix == 1 && (parts & SJVP_BWD_COL) && (HD != 128 || HAS_G);
         if (rc == SJVP_OK && p.rowfix != 0 && !rides)
             rc = launch(bwd_row16_kernel<T, HD, XR, HAS_DO, HAS_G, OCC, 2>, grid, smem, stream, p, kXThreads16);
     }
@@ -39,8 +41,15 @@ int pair_mode(const BwdParams& p, int BH, int parts, hipStream_t stream) {
         // eight waves: wave pairs share 16 keys, split the score-side tiles by query tile and the
         // gradients by head-dimension half (one launch, nothing computed twice)
         constexpr int PR = SJVP_COL16P_RING;  // ring depths 2, 3, 4 measure the same (the kernel is issue-bound)
-        return launch(bwd_col16p_kernel<T, HD, PR, HAS_DO, HAS_G>, grid, Col16pSmem<HD, PR, HAS_DO, HAS_G>::bytes,
-                      stream, p, kThreads16);
+        using PS = Col16pSmem<HD, PR, HAS_DO, HAS_G>;
+        if (rides) {
+            BwdParams pr = p;
+            pr.col_workgroups = grid;
+            constexpr int smem = PS::bytes > Row16Smem<HD, XR, HAS_G>::bytes ? PS::bytes : Row16Smem<HD, XR, HAS_G>::bytes;
+            return launch(bwd_col16p_repair_kernel<T, HD, PR, XR, HAS_DO, HAS_G>, grid + BH * (p.Lr / kXOwned16), smem,
+                          stream, pr, kThreads16);
+        }
+        return launch(bwd_col16p_kernel<T, HD, PR, HAS_DO, HAS_G>, grid, PS::bytes, stream, p, kThreads16);
     } else {
         if (rides) {
             BwdParams pr = p;
