@@ -109,8 +109,7 @@ int sjvp_bwd(const void* q, const void* k, const void* v, const void* tq, const 
  * so that a profiler or benchmark can time the two launches separately.  SJVP_BWD_COL alone is only
  * valid on a workspace that an earlier SJVP_BWD_ROW launch with the same arguments has filled.  (The second
  * pass of the row-owned kernel, see sjvp_set_row_sum_repair, belongs to SJVP_BWD_ROW; with SJVP_BWD_ALL its
- * workgroups are appended to the column-owned launch where the two kernels' workgroups have one size, D <= 64,
- * since it depends on the first row-owned launch only.)
+ * workgroups are appended to the column-owned launch, since it depends on the first row-owned launch only.)
  */
 enum sjvp_bwd_part { SJVP_BWD_ROW = 1, SJVP_BWD_COL = 2, SJVP_BWD_ALL = 3 };
 int sjvp_bwd_parts(int parts, const void* q, const void* k, const void* v, const void* tq,
